@@ -1,0 +1,351 @@
+/*
+ * CPU oracle for the FP8 skinny-GEMM path.  TEST INFRASTRUCTURE ONLY: see
+ * sg_oracle.h for who may call it and for the reference lines each function
+ * restates.
+ */
+#include "sg_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+/* ------------------------------------------------------------------------ */
+/* OCP E4M3 ("e4m3fn"): 1 sign, 4 exponent (bias 7), 3 mantissa bits.       */
+/* No infinities; S.1111.111 is NaN; largest finite is S.1111.110 = 448.    */
+/* ------------------------------------------------------------------------ */
+float orc_e4m3_decode(uint8_t code) {
+    int s = code >> 7, e = (code >> 3) & 0xf, m = code & 7;
+    float v;
+    if (e == 0xf && m == 7) return u2f(0x7fc00000u | ((uint32_t)s << 31));
+    if (e == 0) v = ldexpf((float)m, -9);               /* subnormal: m/8 * 2^-6 */
+    else        v = ldexpf((float)(8 + m), e - 10);     /* (1+m/8) * 2^(e-7)     */
+    return s ? -v : v;
+}
+
+uint8_t orc_e4m3_encode(float x) {
+    uint32_t u = f2u(x);
+    uint8_t sign = (uint8_t)((u >> 24) & 0x80);
+    uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return sign | 0x7f;            /* NaN */
+    if (a >= 0x43e80000u) return sign | 0x7e;           /* |x| >= 464 (incl. inf): saturate to 448 */
+    if (a < 0x3c800000u) {                              /* |x| < 2^-6: subnormal grid, step 2^-9 */
+        /* rintf honours the default round-to-nearest-even mode; result 0..8, and 8 is
+           exactly the code of the smallest normal */
+        float q = rintf(u2f(a) * 512.0f);
+        return sign | (uint8_t)q;
+    }
+    /* normal: round the 23-bit mantissa to 3 bits, ties to even, carry may bump the exponent */
+    uint32_t r = a + 0x7ffffu + ((a >> 20) & 1u);
+    uint32_t code = (r >> 20) - ((127u - 7u) << 3);
+    if (code > 0x7e) code = 0x7e;
+    return sign | (uint8_t)code;
+}
+
+uint16_t orc_bf16_from_f32(float x) {
+    uint32_t u = f2u(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+void orc_e4m3_decode_n(const uint8_t* q, float* out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = orc_e4m3_decode(q[i]);
+}
+void orc_e4m3_encode_n(const float* x, uint8_t* out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = orc_e4m3_encode(x[i]);
+}
+void orc_bf16_from_f32_n(const float* x, uint16_t* out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = orc_bf16_from_f32(x[i]);
+}
+void orc_bf16_to_f32_n(const uint16_t* h, float* out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = orc_bf16_to_f32(h[i]);
+}
+
+static void build_lut(float lut[256]) {
+    for (int i = 0; i < 256; i++) lut[i] = orc_e4m3_decode((uint8_t)i);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Counter-based generator: splitmix64 finaliser over (seed, stream, index). */
+/* ------------------------------------------------------------------------ */
+static inline uint64_t mix64(uint64_t z) {
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+
+uint64_t orc_rng_u64(uint64_t seed, uint64_t stream_id, uint64_t i) {
+    uint64_t key = mix64(seed + 0x9e3779b97f4a7c15ull) ^ mix64(stream_id * 0xd1b54a32d192ed03ull + 0x2545f4914f6cdd1dull);
+    return mix64(key + (i + 1) * 0x9e3779b97f4a7c15ull);
+}
+
+static inline double normal_at(uint64_t seed, uint64_t stream_id, uint64_t i) {
+    /* Box-Muller on two 53-bit uniforms; u1 in (0,1] so the log is finite */
+    double u1 = (double)((orc_rng_u64(seed, stream_id, 2 * i) >> 11) + 1) * 0x1.0p-53;
+    double u2 = (double)(orc_rng_u64(seed, stream_id, 2 * i + 1) >> 11) * 0x1.0p-53;
+    return sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2);
+}
+
+void orc_fill_normal_f32(float* out, size_t n, uint64_t seed, uint64_t stream_id) {
+#pragma omp parallel for schedule(static)
+    for (long long i = 0; i < (long long)n; i++) out[i] = (float)normal_at(seed, stream_id, (uint64_t)i);
+}
+
+void orc_fill_uniform_f32(float* out, size_t n, uint64_t seed, uint64_t stream_id, float lo, float hi) {
+#pragma omp parallel for schedule(static)
+    for (long long i = 0; i < (long long)n; i++) {
+        double u = (double)(orc_rng_u64(seed, stream_id, (uint64_t)i) >> 11) * 0x1.0p-53;
+        out[i] = (float)(lo + (hi - lo) * u);
+    }
+}
+
+void orc_fill_normal_bf16_outliers(uint16_t* out, size_t n, uint64_t seed, uint64_t stream_id,
+                                   double frac, float mag) {
+#pragma omp parallel for schedule(static)
+    for (long long i = 0; i < (long long)n; i++)
+        out[i] = orc_bf16_from_f32((float)normal_at(seed, stream_id, (uint64_t)i));
+    size_t draws = (size_t)floor(frac * (double)n);
+    uint16_t pos = orc_bf16_from_f32(mag), neg = orc_bf16_from_f32(-mag);
+    for (size_t j = 0; j < draws; j++) {           /* sequential: a later draw overwrites an earlier one */
+        uint64_t r = orc_rng_u64(seed, stream_id + 0x100000000ull, j);
+        out[(r >> 1) % n] = (r & 1) ? neg : pos;
+    }
+}
+
+/* ------------------------------------------------------------------------ */
+float orc_absmax_f32(const float* x, size_t n) {
+    float m = 0.0f;
+    for (size_t i = 0; i < n; i++) { float a = fabsf(x[i]); if (a > m) m = a; }
+    return m;
+}
+
+float orc_quantize_tensor(const float* x, uint8_t* q, size_t n) {
+    float amax = orc_absmax_f32(x, n);
+    float scale = (amax == 0.0f) ? 1.0f : amax / 448.0f;
+#pragma omp parallel for schedule(static)
+    for (long long i = 0; i < (long long)n; i++) q[i] = orc_e4m3_encode(x[i] / scale);
+    return scale;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Dense GEMM.  Loop order, "scale once after the K sum", and "cast last"    */
+/* follow projects/skinny_gemm/test.cu:23-38.                                */
+/* ------------------------------------------------------------------------ */
+void orc_gemm_ref(const uint8_t* A, const uint8_t* B, uint16_t* D, float scale,
+                  int m, int n, int k, int b_stride) {
+    for (int i = 0; i < m; i++) {
+        for (int j = 0; j < n; j++) {
+            float acc = 0.0f;
+            const uint8_t* a = A + (size_t)i * k;
+            const uint8_t* b = B + (size_t)j * b_stride;
+            for (int l = 0; l < k; l++) acc += orc_e4m3_decode(a[l]) * orc_e4m3_decode(b[l]);
+            D[(size_t)i * n + j] = orc_bf16_from_f32(acc * scale);
+        }
+    }
+}
+
+static void gemm_rows_f32(const uint8_t* A, const uint8_t* B, float* accs, const float* lut,
+                          int m, int k, int b_stride, int j, const float* Adec) {
+    (void)A;
+    const uint8_t* b = B + (size_t)j * b_stride;
+    for (int i = 0; i < m; i++) {
+        const float* a = Adec + (size_t)i * k;
+        float acc = 0.0f;
+        for (int l = 0; l < k; l++) acc += a[l] * lut[b[l]];
+        accs[i] = acc;
+    }
+}
+
+void orc_gemm_f32(const uint8_t* A, const uint8_t* B, float* D, float scale,
+                  int m, int n, int k, int b_stride) {
+    float lut[256];
+    build_lut(lut);
+    float* Adec = (float*)malloc((size_t)m * k * sizeof(float));
+    for (size_t i = 0; i < (size_t)m * k; i++) Adec[i] = lut[A[i]];
+#pragma omp parallel
+    {
+        float* accs = (float*)malloc((size_t)m * sizeof(float));
+#pragma omp for schedule(static)
+        for (int j = 0; j < n; j++) {
+            gemm_rows_f32(A, B, accs, lut, m, k, b_stride, j, Adec);
+            for (int i = 0; i < m; i++) D[(size_t)i * n + j] = accs[i] * scale;
+        }
+        free(accs);
+    }
+    free(Adec);
+}
+
+void orc_gemm_omp(const uint8_t* A, const uint8_t* B, uint16_t* D, float scale,
+                  int m, int n, int k, int b_stride) {
+    float* tmp = (float*)malloc((size_t)m * n * sizeof(float));
+    orc_gemm_f32(A, B, tmp, scale, m, n, k, b_stride);
+    for (size_t i = 0; i < (size_t)m * n; i++) D[i] = orc_bf16_from_f32(tmp[i]);
+    free(tmp);
+}
+
+void orc_gemm_f64(const uint8_t* A, const uint8_t* B, double* D, double scale,
+                  int m, int n, int k, int b_stride) {
+    float lut[256];
+    build_lut(lut);
+#pragma omp parallel for schedule(static)
+    for (int j = 0; j < n; j++) {
+        const uint8_t* b = B + (size_t)j * b_stride;
+        for (int i = 0; i < m; i++) {
+            const uint8_t* a = A + (size_t)i * k;
+            double acc = 0.0;
+            for (int l = 0; l < k; l++) acc += (double)lut[a[l]] * (double)lut[b[l]];
+            D[(size_t)i * n + j] = acc * scale;
+        }
+    }
+}
+
+int orc_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ------------------------------------------------------------------------ */
+/* 2:4 structured sparsity                                                   */
+/* ------------------------------------------------------------------------ */
+void orc_prune24_f32(float* B, int n, int k) {
+#pragma omp parallel for schedule(static)
+    for (long long g = 0; g < (long long)n * (k / 4); g++) {
+        float* p = B + 4 * g;
+        int i0 = -1, i1 = -1;
+        /* largest |x|, then second largest; strict '>' keeps the lower index on ties */
+        for (int i = 0; i < 4; i++) if (i0 < 0 || fabsf(p[i]) > fabsf(p[i0])) i0 = i;
+        for (int i = 0; i < 4; i++) if (i != i0 && (i1 < 0 || fabsf(p[i]) > fabsf(p[i1]))) i1 = i;
+        for (int i = 0; i < 4; i++) if (i != i0 && i != i1) p[i] = 0.0f;
+    }
+}
+
+int orc_compress24(const uint8_t* B, uint8_t* vals, uint8_t* meta, int n, int k) {
+    size_t groups = (size_t)n * (k / 4);
+    int bad = 0;
+    memset(meta, 0, groups / 2 + (groups & 1));
+    for (size_t g = 0; g < groups; g++) {
+        const uint8_t* p = B + 4 * g;
+        int idx[2], cnt = 0;
+        for (int i = 0; i < 4; i++) {
+            if ((p[i] & 0x7f) != 0) { if (cnt < 2) idx[cnt] = i; cnt++; }
+        }
+        if (cnt > 2) { bad = 1; cnt = 2; }
+        /* pad with the lowest indices not yet used, then sort */
+        for (int i = 0; i < 4 && cnt < 2; i++) {
+            if (cnt == 1 && idx[0] == i) continue;
+            idx[cnt++] = i;
+        }
+        if (idx[0] > idx[1]) { int t = idx[0]; idx[0] = idx[1]; idx[1] = t; }
+        vals[2 * g] = p[idx[0]];
+        vals[2 * g + 1] = p[idx[1]];
+        uint8_t nib = (uint8_t)(idx[0] | (idx[1] << 2));
+        meta[g >> 1] |= (uint8_t)(nib << (4 * (g & 1)));
+    }
+    return bad ? -1 : 0;
+}
+
+void orc_decompress24(const uint8_t* vals, const uint8_t* meta, uint8_t* B, int n, int k) {
+    size_t groups = (size_t)n * (k / 4);
+    memset(B, 0, groups * 4);
+    for (size_t g = 0; g < groups; g++) {
+        uint8_t nib = (meta[g >> 1] >> (4 * (g & 1))) & 0xf;
+        B[4 * g + (nib & 3)] = vals[2 * g];
+        B[4 * g + (nib >> 2)] = vals[2 * g + 1];
+    }
+}
+
+void orc_gemm_sparse24_omp(const uint8_t* A, const uint8_t* vals, const uint8_t* meta,
+                           uint16_t* D, float scale, int m, int n, int k) {
+    uint8_t* B = (uint8_t*)malloc((size_t)n * k);
+    orc_decompress24(vals, meta, B, n, k);
+    orc_gemm_omp(A, B, D, scale, m, n, k, k);
+    free(B);
+}
+
+/* ------------------------------------------------------------------------ */
+/* per-row FP8 codec                                                         */
+/* ------------------------------------------------------------------------ */
+void orc_fp8_encode_rows(const uint16_t* X, uint8_t* Q, float* scales, int rows, int cols) {
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; r++) {
+        const uint16_t* x = X + (size_t)r * cols;
+        float amax = 0.0f;
+        for (int c = 0; c < cols; c++) { float a = fabsf(orc_bf16_to_f32(x[c])); if (a > amax) amax = a; }
+        float s = (amax == 0.0f) ? 1.0f : amax / 448.0f;
+        scales[r] = s;
+        for (int c = 0; c < cols; c++) Q[(size_t)r * cols + c] = orc_e4m3_encode(orc_bf16_to_f32(x[c]) / s);
+    }
+}
+
+void orc_fp8_decode_rows(const uint8_t* Q, const float* scales, uint16_t* Y, int rows, int cols) {
+    float lut[256];
+    build_lut(lut);
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++)
+            Y[(size_t)r * cols + c] = orc_bf16_from_f32(lut[Q[(size_t)r * cols + c]] * scales[r]);
+}
+
+void orc_fp8_reduce_rows(const uint8_t* Q, const float* scales, uint16_t* Y,
+                         int nbuf, int rows, int cols) {
+    float lut[256];
+    build_lut(lut);
+    size_t plane = (size_t)rows * cols;
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            float acc = 0.0f;
+            for (int b = 0; b < nbuf; b++)
+                acc += lut[Q[b * plane + (size_t)r * cols + c]] * scales[(size_t)b * rows + r];
+            Y[(size_t)r * cols + c] = orc_bf16_from_f32(acc);
+        }
+}
+
+/* projects/tiled_sum_reduce/test.cu:5-26 */
+void orc_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n) {
+    size_t mn = (size_t)m * n;
+    for (size_t i = 0; i < mn; i++) D[i] = 0.0f;
+    for (int ib = 0; ib < b; ib++) {
+        for (size_t i = 0; i < mn; i++) D[i] += A[i] + B[i];
+        A += mn;
+        B += mn;
+    }
+}
+
+/* projects/skinny_gemm/test.cu:94-107 */
+void orc_delta_metrics_bf16(const uint16_t* got, const uint16_t* ref, size_t n,
+                            float* max_delta, float* total_delta) {
+    float mx = 0.0f, sum = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        float d = fabsf(orc_bf16_to_f32(got[i]) - orc_bf16_to_f32(ref[i]));
+        sum += d;
+        if (d > mx || d != d) mx = d;
+    }
+    *max_delta = mx;
+    *total_delta = sum;
+}
+
+double orc_max_rel_err_bf16(const uint16_t* got, const uint16_t* ref, size_t n) {
+    double ss = 0.0;
+    for (size_t i = 0; i < n; i++) { double r = orc_bf16_to_f32(ref[i]); ss += r * r; }
+    double floor_ = 1e-2 * sqrt(ss / (double)(n ? n : 1));
+    double worst = 0.0;
+    for (size_t i = 0; i < n; i++) {
+        double r = orc_bf16_to_f32(ref[i]), g = orc_bf16_to_f32(got[i]);
+        double den = fabs(r) > floor_ ? fabs(r) : floor_;
+        double e = (den > 0.0) ? fabs(g - r) / den : fabs(g - r);
+        if (e > worst || e != e) worst = e;
+    }
+    return worst;
+}

@@ -1,0 +1,242 @@
+"""Pins the oracle's GEMM, 2:4 and per-row codec functions.
+
+The GEMM restates projects/skinny_gemm/test.cu:7-39 (sequential fp32 sum over k, scale
+once, cast last) for OCP E4M3 operands and bf16 output.  Because products of two E4M3
+values are exact in fp32, the only freedom is the summation order; the checks below are
+chosen so that a dropped term, a transposed operand, a wrong stride or a misplaced scale
+fails at least one of them.  Independent arithmetic comes from numpy / torch, never from
+the oracle itself.
+"""
+import numpy as np
+import pytest
+import torch
+
+
+def _dec(q):
+    """Independent decode: torch's float8_e4m3fn CPU cast."""
+    return torch.from_numpy(np.ascontiguousarray(q)).view(torch.float8_e4m3fn).double().numpy()
+
+
+def _bf16(x):
+    return torch.from_numpy(np.asarray(x, dtype=np.float32)).bfloat16().view(torch.int16).numpy().view(np.uint16)
+
+
+def _rand_codes(rng, shape):
+    q = rng.integers(0, 256, size=shape, dtype=np.uint8)
+    q[(q & 0x7F) == 0x7F] = 0x38
+    return q
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 2, 8), (3, 5, 16), (8, 64, 64), (17, 10, 48)])
+def test_tiny_vs_fp64_numpy(oracle, m, n, k):
+    rng = np.random.default_rng(m * 1000 + n * 10 + k)
+    A, B = _rand_codes(rng, (m, k)), _rand_codes(rng, (n, k))
+    # keep magnitudes modest so fp32 sums are near-exact and bf16 rounding is decisive
+    A &= 0xBF
+    B &= 0xBF
+    scale = np.float32(0.37)
+    truth = (_dec(A) @ _dec(B).T)
+    got64 = oracle.gemm_f64(A, B, 1.0)
+    assert np.array_equal(got64, truth)                      # exact in fp64 for these sizes
+    got = oracle.bf16_to_f32(oracle.gemm_ref(A, B, scale))
+    want = truth * float(scale)
+    assert np.allclose(got, want, rtol=2 ** -8, atol=1e-30)
+    assert np.array_equal(oracle.gemm_ref(A, B, scale), oracle.gemm_omp(A, B, scale))
+
+
+def test_sequential_order_is_what_is_restated(oracle):
+    """fp32 left-to-right accumulation, reproduced with numpy float32 scalars."""
+    rng = np.random.default_rng(5)
+    m, n, k = 2, 3, 512
+    A, B = _rand_codes(rng, (m, k)), _rand_codes(rng, (n, k))
+    da, db = _dec(A).astype(np.float32), _dec(B).astype(np.float32)
+    scale = np.float32(1.25e-3)
+    want = np.empty((m, n), np.float32)
+    for i in range(m):
+        for j in range(n):
+            acc = np.float32(0)
+            for l in range(k):
+                acc = np.float32(acc + np.float32(da[i, l] * db[j, l]))
+            want[i, j] = np.float32(acc * scale)
+    assert np.array_equal(oracle.gemm_f32(A, B, scale), want)
+    assert np.array_equal(oracle.gemm_ref(A, B, scale), _bf16(want))
+
+
+def test_invariants(oracle):
+    rng = np.random.default_rng(11)
+    m, n, k = 8, 32, 64
+    A = _rand_codes(rng, (m, k))
+    one = 0x38  # 1.0
+    # one-hot B rows select single A columns: D[i, j] = dec(A[i, j]) * scale exactly
+    B = np.zeros((n, k), np.uint8)
+    for j in range(n):
+        B[j, (3 * j + 1) % k] = one
+    scale = np.float32(0.5)
+    got = oracle.bf16_to_f32(oracle.gemm_ref(A, B, scale))
+    want = np.stack([_dec(A)[:, (3 * j + 1) % k] for j in range(n)], axis=1) * 0.5
+    assert np.array_equal(got, want.astype(np.float32))
+    # zero A -> zero D
+    assert not oracle.gemm_ref(np.zeros_like(A), _rand_codes(rng, (n, k)), scale).any()
+    # all ones, K = 4096 -> exactly 4096 * s
+    K = 4096
+    ones_a, ones_b = np.full((2, K), one, np.uint8), np.full((4, K), one, np.uint8)
+    assert np.all(oracle.gemm_f32(ones_a, ones_b, 0.25) == 1024.0)
+    # scale is applied once, after the sum
+    Bq = _rand_codes(rng, (n, k))
+    d1 = oracle.gemm_f32(A, Bq, 1.0)
+    d2 = oracle.gemm_f32(A, Bq, 2.0)
+    assert np.array_equal(d2, d1 * 2)
+
+
+def test_b_stride_and_transposition(oracle):
+    rng = np.random.default_rng(3)
+    m, n, k, bs = 4, 6, 32, 48
+    A = _rand_codes(rng, (m, k))
+    Bfull = np.full((n, bs), 0x7F, np.uint8)  # NaN padding: reading it poisons the result
+    Bfull[:, :k] = _rand_codes(rng, (n, k))
+    Dp = np.empty((m, n), np.float32)
+    import ctypes as C
+    oracle._lib.orc_gemm_f32(oracle._p(A), oracle._p(Bfull), oracle._p(Dp), 1.0, m, n, k, bs)
+    want = _dec(A) @ _dec(Bfull[:, :k]).T
+    assert np.allclose(Dp, want, rtol=1e-5, atol=1e-5)
+    assert Dp.shape == (m, n) and not np.isnan(Dp).any()
+
+
+def test_config1_against_torch_fp64(oracle):
+    """BASELINE config 1 (8 x 4096 x 4096, seed 0): oracle vs torch fp64 matmul of the dequantised operands."""
+    a8, b8, scale = oracle.make_gemm_operands(8, 4096, 4096, seed=0)
+    truth = torch.from_numpy(_dec(a8)) @ torch.from_numpy(_dec(b8)).T * float(scale)
+    got = oracle.bf16_to_f32(oracle.gemm_omp(a8, b8, scale))
+    rel = oracle.max_rel_err_bf16(oracle.gemm_omp(a8, b8, scale), _bf16(truth.numpy()))
+    assert rel < 1e-2
+    assert np.abs(got - truth.numpy()).max() <= 2 ** -8 * np.abs(truth.numpy()).max() + 1e-3
+    # quantisation recipe: absmax maps to +-448
+    assert (a8 & 0x7F).max() == 0x7E and (b8 & 0x7F).max() == 0x7E
+    # reference loop == all-core loop on a slice
+    assert np.array_equal(oracle.gemm_ref(a8[:2], b8[:64], scale), oracle.gemm_omp(a8[:2], b8[:64], scale))
+
+
+def test_max_rel_err_metric(oracle):
+    ref = _bf16(np.array([1.0, -2.0, 0.0, 4.0], np.float32))
+    got = _bf16(np.array([1.0, -2.0, 0.0, 4.0], np.float32))
+    assert oracle.max_rel_err_bf16(got, ref) == 0.0
+    got2 = _bf16(np.array([1.0, -2.0, 0.0, 4.5], np.float32))
+    assert abs(oracle.max_rel_err_bf16(got2, ref) - 0.125) < 1e-12
+    # small |ref| is floored at 1e-2 * rms(ref)
+    rms = np.sqrt((1 + 4 + 0 + 16) / 4)
+    got3 = _bf16(np.array([1.0, -2.0, 0.015625, 4.0], np.float32))
+    assert abs(oracle.max_rel_err_bf16(got3, ref) - 0.015625 / (1e-2 * rms)) < 1e-9
+    mx, tot = oracle.delta_metrics_bf16(got2, ref)
+    assert mx == 0.5 and tot == 0.5
+
+
+# ---- 2:4 ---------------------------------------------------------------------------
+def test_prune24_independent(oracle):
+    rng = np.random.default_rng(9)
+    B = rng.standard_normal((16, 64)).astype(np.float32)
+    B[0, :4] = [1.0, -1.0, 1.0, 0.5]      # tie: keep indices 0 and 1
+    B[1, :4] = [0.0, 0.0, 0.0, 0.0]
+    B[2, :4] = [2.0, 3.0, 3.0, 2.0]       # keep 1, 2
+    got = oracle.prune24(B)
+    g = B.reshape(-1, 4)
+    # stable argsort of -|x| keeps the lower index first on ties
+    order = np.argsort(-np.abs(g), axis=1, kind="stable")[:, :2]
+    want = np.zeros_like(g)
+    rows = np.arange(g.shape[0])[:, None]
+    want[rows, order] = g[rows, order]
+    assert np.array_equal(got.reshape(-1, 4), want)
+    assert np.array_equal(got[0, :4], [1.0, -1.0, 0.0, 0.0])
+    assert np.array_equal(got[2, :4], [0.0, 3.0, 3.0, 0.0])
+    assert ((got.reshape(-1, 4) != 0).sum(1) <= 2).all()
+
+
+def test_compress24_known_answer_and_roundtrip(oracle):
+    B = np.zeros((1, 16), np.uint8)
+    B[0, 0:4] = [0x38, 0, 0, 0x40]     # kept idx 0,3 -> nibble 0b1100 = 0xC
+    B[0, 4:8] = [0, 0x39, 0x3A, 0]     # kept idx 1,2 -> nibble 0b1001 = 0x9
+    B[0, 8:12] = [0, 0, 0, 0x41]       # one non-zero at 3 -> pad with 0 -> (0,3) -> 0xC, vals (0, 0x41)
+    B[0, 12:16] = [0, 0, 0, 0]         # empty -> (0,1) -> 0x4
+    vals, meta = oracle.compress24(B)
+    assert vals.tolist() == [[0x38, 0x40, 0x39, 0x3A, 0x00, 0x41, 0x00, 0x00]]
+    assert meta.tolist() == [[0x9C, 0x4C]]
+    assert np.array_equal(oracle.decompress24(vals, meta), B)
+    with pytest.raises(ValueError):
+        oracle.compress24(np.full((1, 8), 0x38, np.uint8))
+    a8, vals, meta, b8, scale = oracle.make_sparse24_operands(8, 64, 256, seed=0)
+    assert vals.shape == (64, 128) and meta.shape == (64, 32)
+    assert np.array_equal(oracle.decompress24(vals, meta), b8)
+    assert np.array_equal(oracle.gemm_sparse24(a8, vals, meta, scale), oracle.gemm_omp(a8, b8, scale))
+    # every group's first index is below its second
+    nib = np.stack([meta & 0xF, meta >> 4], axis=-1).reshape(64, -1)
+    assert ((nib & 3) < (nib >> 2)).all()
+
+
+# ---- per-row codec -------------------------------------------------------------------
+def test_codec_against_torch(oracle):
+    rows, cols = 64, 512
+    X = oracle.normal_bf16_outliers((rows, cols), seed=0, stream_id=3, frac=0.001, mag=50.0)
+    X[5] = 0  # all-zero row: scale is defined as 1
+    xt = torch.from_numpy(X.view(np.int16)).view(torch.bfloat16).float()
+    amax = xt.abs().amax(dim=1)
+    scale = torch.where(amax == 0, torch.ones_like(amax), amax / 448.0)
+    want_q = (xt / scale[:, None]).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    Q, s = oracle.fp8_encode_rows(X)
+    assert np.array_equal(s, scale.numpy())
+    assert np.array_equal(Q, want_q)
+    assert s[5] == 1.0 and not Q[5].any()
+    # outliers present and mapped to +-448 in rows that contain one
+    has = (np.abs(xt.numpy()) == 50.0).any(axis=1)
+    assert has.any() and ((Q[has] & 0x7F).max(axis=1) == 0x7E).all()
+    # decode
+    want_y = (torch.from_numpy(want_q).view(torch.float8_e4m3fn).float() * scale[:, None]).bfloat16()
+    Y = oracle.fp8_decode_rows(Q, s)
+    assert np.array_equal(Y, want_y.view(torch.int16).numpy().view(np.uint16))
+
+
+def test_reduce_rows(oracle):
+    nbuf, rows, cols = 8, 16, 256
+    Qs, Ss = [], []
+    for i in range(nbuf):
+        X = oracle.normal_bf16_outliers((rows, cols), seed=i, stream_id=3)
+        Q, s = oracle.fp8_encode_rows(X)
+        Qs.append(Q)
+        Ss.append(s)
+    Q, S = np.stack(Qs), np.stack(Ss)
+    got = oracle.fp8_reduce_rows(Q, S)
+    # independent fp32 in-order sum with torch
+    acc = torch.zeros(rows, cols)
+    for i in range(nbuf):
+        acc = acc + torch.from_numpy(Q[i]).view(torch.float8_e4m3fn).float() * torch.from_numpy(S[i])[:, None]
+    assert np.array_equal(got, acc.bfloat16().view(torch.int16).numpy().view(np.uint16))
+    truth = sum(_dec(Q[i]) * S[i].astype(np.float64)[:, None] for i in range(nbuf))
+    assert oracle.max_rel_err_bf16(got, _bf16(truth)) < 1e-2
+    # nbuf = 1 reduces to decode
+    assert np.array_equal(oracle.fp8_reduce_rows(Q[:1], S[:1]), oracle.fp8_decode_rows(Q[0], S[0]))
+
+
+def test_tiled_sum_reduce(oracle):
+    rng = np.random.default_rng(2)
+    A = rng.random((5, 8, 64), dtype=np.float32) - 0.5
+    B = rng.random((5, 8, 64), dtype=np.float32) - 0.5
+    want = np.zeros((8, 64), np.float32)
+    for b in range(5):
+        want = want + (A[b] + B[b])
+    assert np.array_equal(oracle.tiled_sum_reduce(A, B), want)
+
+
+# ---- generator -------------------------------------------------------------------------
+def test_generator(oracle):
+    x = oracle.normal_f32((1 << 20,), 0, 1)
+    assert abs(float(x.mean())) < 5e-3 and abs(float(x.std()) - 1.0) < 5e-3
+    assert abs(float((x ** 4).mean()) - 3.0) < 0.05
+    assert np.array_equal(x[:1000], oracle.normal_f32((1000,), 0, 1))       # counter based
+    assert not np.array_equal(x[:1000], oracle.normal_f32((1000,), 1, 1))
+    assert not np.array_equal(x[:1000], oracle.normal_f32((1000,), 0, 2))
+    u = oracle.uniform_f32((1 << 18,), 0, 5, -1.0, 1.0)
+    assert u.min() >= -1.0 and u.max() < 1.0 and abs(float(u.mean())) < 5e-3
+    n = 1 << 20
+    X = oracle.normal_bf16_outliers((n,), 0, 3, 0.001, 50.0)
+    xf = oracle.bf16_to_f32(X)
+    cnt = int((np.abs(xf) == 50.0).sum())
+    assert 0.99 * int(0.001 * n) <= cnt <= int(0.001 * n)
+    assert (xf == 50.0).any() and (xf == -50.0).any()
