@@ -1,0 +1,133 @@
+/*
+ * sgemm.h - C ABI of the MI355X (gfx950) FP8 skinny-GEMM library, libsgemm.so.
+ *
+ * Every entry point is enqueue-only: it validates its arguments on the host, launches
+ * on the given HIP stream (a hipStream_t passed as void*; NULL is the default stream)
+ * and returns without synchronising.  All data pointers are DEVICE pointers owned by
+ * the caller.  Nothing here calls exit(); failures come back as SgReturnCode values.
+ *
+ * Formats: "fp8" is OCP E4M3 (one byte, 0x7f/0xff NaN, max 448) - the format gfx950
+ * MFMA decodes - not the E4M3 FNUZ of gfx942.  "bf16" is the upper half of an IEEE
+ * binary32, rounded to nearest even.  Weights B are N x K, K contiguous, row stride
+ * b_stride bytes; activations A are M x K row-major; outputs D are M x N row-major.
+ *
+ * Differences from the reference launchers that a caller must know:
+ *   - D is OVERWRITTEN (the reference accumulates with atomics into a pre-zeroed D);
+ *   - D is bf16 (the reference writes fp16 or fp32);
+ *   - split-K partial sums are reduced in fp32 in a fixed order, so results are
+ *     bit-reproducible from run to run.
+ *
+ * Reference citations are paths below the reference tree's projects/ directory.
+ */
+#ifndef SGEMM_H
+#define SGEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Codes 0-6 are the reference's SkinnyGemmReturnCode verbatim
+ * (skinny_gemm/skinny_gemm_caller.cu:9-17); codes >= 7 are additions. */
+typedef enum SgReturnCode {
+    SG_SUCCESS = 0,
+    SG_M_ABOVE_WARPTILE_M = 1,             /* kept for numbering; never returned (unused in the reference too) */
+    SG_N_NOT_EVEN = 2,
+    SG_K_NOT_DIVISIBLE_BY_WARPTILE_K = 3,
+    SG_TOO_MANY_WARPS = 4,
+    SG_QSIZE_TOO_SMALL = 5,
+    SG_INVALID_CONFIG = 6,
+    SG_LAUNCH_FAILED = 7,                  /* the HIP runtime refused the launch */
+    SG_BAD_ALIGNMENT = 8,                  /* pointer or stride not 16-byte aligned */
+    SG_BAD_ARGUMENT = 9,                   /* null pointer, non-positive size, ... */
+    SG_WORKSPACE_TOO_SMALL = 10,           /* split-K partials do not fit the workspace */
+    SG_NO_DEVICE = 11                      /* no usable gfx950 device / HIP runtime error at set-up */
+} SgReturnCode;
+
+const char* sg_strerror(int code);
+
+/* Library-owned split-K workspace, one per device, created on first use by a launcher
+ * that needs it (split_k > 1).  sg_init() creates it eagerly for the current device so
+ * that later launches allocate nothing.  Two launches that use split-K concurrently on
+ * different streams of one device share it and therefore must not overlap. */
+int    sg_init(void);
+size_t sg_workspace_bytes(void);
+
+/*
+ * Dense FP8 skinny GEMM:  D[m,n] = bf16( scale[0] * sum_k A[m,k] * B[n,k] ).
+ * Replaces  int skinny_gemm(const fp8*, const fp8*, half*, const float*, int m, int n,
+ * int k, int b_stride, int split_k, int A_producers, int B_producers, int consumers,
+ * int b_lanes, int qsize, int op_m, int ops, hipStream_t)
+ * (skinny_gemm/skinny_gemm_caller.cu:20-43) - same parameter list, same validation
+ * order and return codes (:55-75).  Meaning of the tunables in this library:
+ *   op_m     8, 16 or 32: rows of A covered by one MFMA column block (8 and 16 use one
+ *            16-wide block with unused rows masked, 32 uses two); m above op_m is
+ *            covered by further row tiles, each re-streaming B, as in the reference
+ *            (skinny_gemm/skinny_gemm_kernel.cu:44-46).
+ *   ops      MFMA K-steps per pipeline stage: a stage is WARPTILE_K = (512/op_m)*ops
+ *            bytes of K per weight row; k must be a multiple of it.
+ *   b_lanes  16-row weight tiles that share one activation fragment (1..4).
+ *   qsize    stages kept in flight per wave (register ring depth) / LDS ring slots.
+ *   A_producers, B_producers, consumers
+ *            wavefront roles of one workgroup, at most 16 in total.  With
+ *            A_producers == 0 and B_producers == 0 every one of the `consumers` waves
+ *            streams its own operands from global memory straight into MFMA registers
+ *            (no LDS hop) and the waves of a workgroup split K among themselves; with
+ *            producers > 0 the operands go through an LDS ring filled by the producer
+ *            waves, as in the reference.
+ *   split_k  K is also split across split_k workgroups; partials meet in the fp32
+ *            workspace and the last workgroup to arrive reduces them in split order.
+ */
+int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                   int m, int n, int k, int b_stride, int split_k,
+                   int A_producers, int B_producers, int consumers,
+                   int b_lanes, int qsize, int op_m, int ops, void* stream);
+
+/* Replaces  int skinny_gemm_fastpath(const fp8* A, const fp8* B, half* D, const float*
+ * scale_tensor, int m, int n, int k)  (skinny_gemm/skinny_gemm_caller.cu:343-405):
+ * b_stride = k, default stream, tunables chosen by the library for the shape instead of
+ * compiled-in #defines (skinny_gemm/core.cu:29-38).  Requires k % 16 == 0 and n even. */
+int sg_skinny_gemm_fastpath(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                            int m, int n, int k);
+
+/* The fastpath with an explicit row stride and stream (what the torch binding passes,
+ * skinny_gemm/skinny_gemm_binding.cu:36-60). */
+int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                        int m, int n, int k, int b_stride, void* stream);
+
+/* The configuration sg_skinny_gemm_auto would use, for logging and tuning drivers.
+ * out[8] = {split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops}. */
+int sg_skinny_gemm_pick(int m, int n, int k, int out[8]);
+
+/* Replaces  template<class out> void async_gemm(const fp8* A, const fp8* B, out* D, int m,
+ * int n, int k)  (async_gemm_sparse/sparse_k.cu:45-69, async_gemm_blanes/sparse_k.cu,
+ * async_gemm_16x16x64/src.cu:55-82): D = A * B^T without a scale, default stream, through
+ * the LDS producer/consumer ring.  The reference prints and exits on a bad shape; these
+ * return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K / SG_BAD_ARGUMENT instead.  D is overwritten. */
+int sg_async_gemm_f32(const uint8_t* A, const uint8_t* B, float* D, int m, int n, int k);
+int sg_async_gemm_bf16(const uint8_t* A, const uint8_t* B, void* D_bf16, int m, int n, int k);
+
+/* Replaces  void tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m,
+ * int n)  (tiled_sum_reduce/src.cu:52-73):  D[m,n] = sum_b (A[b,m,n] + B[b,m,n]), summed
+ * in batch order per element.  Any m, n (the reference needs m % 8 == 0, n % 64 == 0). */
+int sg_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n, void* stream);
+
+/* Per-row FP8 codec - no counterpart in the reference; the local compute on either side
+ * of an FP8 all-reduce exchange.
+ *   encode: scales[r] = absmax(X[r,:]) / 448 (1 if the row is all zero),
+ *           Q[r,c] = e4m3_rne_sat( X[r,c] / scales[r] )                  (bit exact)
+ *   decode: Y[r,c] = bf16( dec(Q[r,c]) * scales[r] )
+ *   reduce: Y[r,c] = bf16( sum_{i<nbuf} dec(Q_i[r,c]) * scales_i[r] ), fp32, buffer order;
+ *           buffer i starts at Q + i*q_buf_stride bytes, scales at scales + i*rows.
+ * cols must be a multiple of 16; X, Q, Y must be 16-byte aligned. */
+int sg_fp8_encode_rows(const void* X_bf16, uint8_t* Q, float* scales, int rows, int cols, void* stream);
+int sg_fp8_decode_rows(const uint8_t* Q, const float* scales, void* Y_bf16, int rows, int cols, void* stream);
+int sg_fp8_reduce_rows(const uint8_t* Q, const float* scales, void* Y_bf16,
+                       int nbuf, size_t q_buf_stride, int rows, int cols, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SGEMM_H */

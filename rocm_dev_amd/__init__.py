@@ -1,0 +1,21 @@
+"""MI355X (gfx950) FP8 skinny-GEMM library: Python host side over the C ABI of libsgemm.so.
+
+The names mirror the reference's launchers (``skinny_gemm``, ``skinny_gemm_fastpath``,
+``async_gemm``, ``tiled_sum_reduce``) and its torch binding class ``HFRK_skinny_gemm``;
+torch is used only for device memory and streams.
+"""
+from .api import (  # noqa: F401
+    HFRK_skinny_gemm,
+    SgError,
+    SgReturnCode,
+    async_gemm,
+    fp8_decode_rows,
+    fp8_encode_rows,
+    fp8_reduce_rows,
+    skinny_gemm,
+    skinny_gemm_fastpath,
+    skinny_gemm_pick,
+    strerror,
+    tiled_sum_reduce,
+)
+from .build import build  # noqa: F401

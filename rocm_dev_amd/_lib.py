@@ -1,0 +1,38 @@
+"""Loads libsgemm.so and declares the C ABI of include/sgemm.h to ctypes.
+
+There is no fallback: if the library has not been built the import fails loudly.
+"""
+import ctypes as C
+import os
+
+from .build import LIB_PATH
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "%s is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+        "or `make -C rocm_dev_amd/csrc`" % LIB_PATH)
+
+lib = C.CDLL(LIB_PATH)
+
+_vp, _i, _sz = C.c_void_p, C.c_int, C.c_size_t
+
+SIGNATURES = {
+    "sg_strerror": (C.c_char_p, [_i]),
+    "sg_init": (_i, []),
+    "sg_workspace_bytes": (_sz, []),
+    "sg_skinny_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "sg_skinny_gemm_fastpath": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
+    "sg_skinny_gemm_auto": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "sg_skinny_gemm_pick": (_i, [_i, _i, _i, C.POINTER(_i * 8)]),
+    "sg_async_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i]),
+    "sg_async_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i]),
+    "sg_tiled_sum_reduce": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sg_fp8_encode_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "sg_fp8_decode_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "sg_fp8_reduce_rows": (_i, [_vp, _vp, _vp, _i, _sz, _i, _i, _vp]),
+}
+
+for _name, (_res, _args) in SIGNATURES.items():
+    _fn = getattr(lib, _name)
+    _fn.restype = _res
+    _fn.argtypes = _args

@@ -1,0 +1,169 @@
+"""Host-side mirror of the reference's launcher and torch-binding surface.
+
+Reference interfaces mirrored (paths below the reference's projects/ directory):
+  skinny_gemm(...)            skinny_gemm/skinny_gemm_caller.cu:20-43
+  skinny_gemm_fastpath(...)   skinny_gemm/skinny_gemm_caller.cu:343-346
+  HFRK_skinny_gemm            skinny_gemm/skinny_gemm_binding.cu:64-100
+  async_gemm(...)             async_gemm_sparse/sparse_k.cu:45-69
+  tiled_sum_reduce(...)       tiled_sum_reduce/src.cu:52-73
+Every function returns the integer return code of the C ABI (0 = success), as the
+reference's launchers do; ``check=True`` raises SgError instead.  Tensors are torch CUDA
+tensors used purely as device buffers: fp8 operands are uint8 or float8_e4m3fn, outputs
+bfloat16 (or float32 for async_gemm), and everything is enqueued on torch's current stream.
+"""
+import enum
+
+import torch
+
+from ._lib import lib
+
+
+class SgReturnCode(enum.IntEnum):
+    SUCCESS = 0
+    M_ABOVE_WARPTILE_M = 1
+    N_NOT_EVEN = 2
+    K_NOT_DIVISIBLE_BY_WARPTILE_K = 3
+    TOO_MANY_WARPS = 4
+    QSIZE_TOO_SMALL = 5
+    INVALID_CONFIG = 6
+    LAUNCH_FAILED = 7
+    BAD_ALIGNMENT = 8
+    BAD_ARGUMENT = 9
+    WORKSPACE_TOO_SMALL = 10
+    NO_DEVICE = 11
+
+
+class SgError(RuntimeError):
+    def __init__(self, code):
+        self.code = int(code)
+        super().__init__("libsgemm: %s (code %d)" % (strerror(code), code))
+
+
+def strerror(code):
+    return lib.sg_strerror(int(code)).decode()
+
+
+def _done(rc, check):
+    if check and rc != 0:
+        raise SgError(rc)
+    return rc
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t, *dtypes):
+    if not t.is_cuda:
+        raise ValueError("expected a CUDA (HIP) tensor")
+    if dtypes and t.dtype not in dtypes:
+        raise ValueError("expected dtype in %s, got %s" % (dtypes, t.dtype))
+    return t.data_ptr()
+
+
+_FP8 = (torch.uint8, torch.float8_e4m3fn)
+
+
+def skinny_gemm(A, B, D, scale_tensor, split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops,
+                b_stride=None, check=False):
+    """D[m,n] = bf16(scale * A[m,k] @ B[n,k]^T) with explicit tunables.  B is [n, k] with row stride b_stride."""
+    m, k = A.shape
+    n = B.shape[0]
+    if b_stride is None:
+        b_stride = B.stride(0)
+    with torch.cuda.device(A.device):
+        rc = lib.sg_skinny_gemm(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
+                                _dev(scale_tensor, torch.float32), m, n, k, b_stride, split_k, A_producers,
+                                B_producers, consumers, b_lanes, qsize, op_m, ops, _stream())
+    return _done(rc, check)
+
+
+def skinny_gemm_fastpath(A, B, D, scale_tensor, check=False):
+    """Library-chosen configuration; B is [n, k] (row stride taken from the tensor)."""
+    m, k = A.shape
+    n = B.shape[0]
+    with torch.cuda.device(A.device):
+        rc = lib.sg_skinny_gemm_auto(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
+                                     _dev(scale_tensor, torch.float32), m, n, k, B.stride(0), _stream())
+    return _done(rc, check)
+
+
+def skinny_gemm_pick(m, n, k):
+    """The tunables the fastpath would use: dict with the reference's parameter names."""
+    import ctypes as C
+    out = (C.c_int * 8)()
+    rc = lib.sg_skinny_gemm_pick(m, n, k, C.byref(out))
+    if rc != 0:
+        raise SgError(rc)
+    names = ("split_k", "A_producers", "B_producers", "consumers", "b_lanes", "qsize", "op_m", "ops")
+    return dict(zip(names, list(out)))
+
+
+class HFRK_skinny_gemm:
+    """Same constructor and method as the reference's torch extension class.
+
+    ``B`` is passed as the reference passes it: a (k, n) *view* of an n x k, K-contiguous
+    weight, so n = B.size(1) and b_stride = B.stride(1) (skinny_gemm_binding.cu:36-39).
+    op_m follows m: 8, 16 or 32 (skinny_gemm_binding.cu:42-45).  D is bfloat16 and is
+    overwritten.
+    """
+
+    def __init__(self, world_size):
+        self.world_size = world_size  # unused, as in the reference
+
+    def skinny_gemm_torch_binding(self, A, B, D, scale_tensor, split_k, A_producers, B_producers, consumers,
+                                  b_lanes, qsize, ops):
+        m, k = A.size(0), A.size(1)
+        n = B.size(1)
+        b_stride = B.stride(1)
+        op_m = 8 if m <= 8 else (16 if m <= 16 else 32)
+        with torch.cuda.device(A.device):
+            return lib.sg_skinny_gemm(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
+                                      _dev(scale_tensor, torch.float32), m, n, k, b_stride, split_k, A_producers,
+                                      B_producers, consumers, b_lanes, qsize, op_m, ops, _stream())
+
+
+def async_gemm(A, B, D, check=False):
+    """D = A @ B^T without a scale on the default stream; D is float32 or bfloat16."""
+    m, k = A.shape
+    n = B.shape[0]
+    with torch.cuda.device(A.device):
+        if D.dtype == torch.float32:
+            rc = lib.sg_async_gemm_f32(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D), m, n, k)
+        else:
+            rc = lib.sg_async_gemm_bf16(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16), m, n, k)
+    return _done(rc, check)
+
+
+def tiled_sum_reduce(A, B, D, check=False):
+    """D[m,n] = sum_b (A[b,m,n] + B[b,m,n]) in fp32, batch order."""
+    b, m, n = A.shape
+    with torch.cuda.device(A.device):
+        rc = lib.sg_tiled_sum_reduce(_dev(A, torch.float32), _dev(B, torch.float32), _dev(D, torch.float32),
+                                     b, m, n, _stream())
+    return _done(rc, check)
+
+
+def fp8_encode_rows(X, Q, scales, check=False):
+    rows, cols = X.shape
+    with torch.cuda.device(X.device):
+        rc = lib.sg_fp8_encode_rows(_dev(X, torch.bfloat16), _dev(Q, *_FP8), _dev(scales, torch.float32),
+                                    rows, cols, _stream())
+    return _done(rc, check)
+
+
+def fp8_decode_rows(Q, scales, Y, check=False):
+    rows, cols = Q.shape
+    with torch.cuda.device(Q.device):
+        rc = lib.sg_fp8_decode_rows(_dev(Q, *_FP8), _dev(scales, torch.float32), _dev(Y, torch.bfloat16),
+                                    rows, cols, _stream())
+    return _done(rc, check)
+
+
+def fp8_reduce_rows(Q, scales, Y, check=False):
+    """Q [nbuf, rows, cols], scales [nbuf, rows] -> Y [rows, cols] bfloat16."""
+    nbuf, rows, cols = Q.shape
+    with torch.cuda.device(Q.device):
+        rc = lib.sg_fp8_reduce_rows(_dev(Q, *_FP8), _dev(scales, torch.float32), _dev(Y, torch.bfloat16),
+                                    nbuf, Q.stride(0), rows, cols, _stream())
+    return _done(rc, check)

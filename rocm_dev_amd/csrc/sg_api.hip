@@ -1,0 +1,284 @@
+// C ABI of libsgemm.so: argument validation, configuration choice and launches.
+// The contract of every entry point is documented in include/sgemm.h.
+#include <mutex>
+
+#include "sg_host.h"
+#include "sg_stream_kernel.h"
+
+namespace sg {
+
+int launch_fp8_encode_rows(const void* X, uint8_t* Q, float* scales, int rows, int cols, hipStream_t stream);
+int launch_fp8_decode_rows(const uint8_t* Q, const float* scales, void* Y, int rows, int cols, hipStream_t stream);
+int launch_fp8_reduce_rows(const uint8_t* Q, const float* scales, void* Y, int nbuf, size_t q_buf_stride, int rows,
+                           int cols, hipStream_t stream);
+int launch_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n, hipStream_t stream);
+
+// ---- per-device state -------------------------------------------------------------------
+constexpr int kMaxDevices = 16;
+constexpr size_t kPartialBytes = 64u << 20;  // fp32 split-K partials
+constexpr size_t kCounters = 1u << 18;       // arrival counters (one per output tile)
+
+static std::mutex g_mutex;
+static Workspace g_ws[kMaxDevices];
+static DeviceInfo g_dev[kMaxDevices];
+static bool g_dev_known[kMaxDevices];
+
+static int current_device(int* dev) {
+    if (hipGetDevice(dev) != hipSuccess || *dev < 0 || *dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return SG_NO_DEVICE;
+    }
+    return SG_SUCCESS;
+}
+
+int get_device_info(DeviceInfo** out) {
+    int dev;
+    if (int rc = current_device(&dev)) return rc;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (!g_dev_known[dev]) {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            return SG_NO_DEVICE;
+        }
+        g_dev[dev].cu_count = prop.multiProcessorCount;
+        g_dev[dev].lds_per_block = (int)prop.sharedMemPerBlock;
+        g_dev[dev].is_gfx950 = std::string(prop.gcnArchName).rfind("gfx950", 0) == 0;
+        g_dev_known[dev] = true;
+    }
+    *out = &g_dev[dev];
+    return g_dev[dev].is_gfx950 ? SG_SUCCESS : SG_NO_DEVICE;
+}
+
+int get_workspace(Workspace** out) {
+    int dev;
+    if (int rc = current_device(&dev)) return rc;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    Workspace& w = g_ws[dev];
+    if (!w.partials) {
+        void* p = nullptr;
+        void* c = nullptr;
+        if (hipMalloc(&p, kPartialBytes) != hipSuccess || hipMalloc(&c, kCounters * sizeof(unsigned)) != hipSuccess ||
+            hipMemset(c, 0, kCounters * sizeof(unsigned)) != hipSuccess) {
+            (void)hipGetLastError();
+            if (p) (void)hipFree(p);
+            if (c) (void)hipFree(c);
+            return SG_NO_DEVICE;
+        }
+        w.partials = static_cast<float*>(p);
+        w.counters = static_cast<unsigned*>(c);
+        w.partial_bytes = kPartialBytes;
+        w.n_counters = kCounters;
+    }
+    *out = &w;
+    return SG_SUCCESS;
+}
+
+// ---- streaming kernel dispatch ----------------------------------------------------------
+struct StreamConfig {
+    int mt, rg, ku, depth, waves, split_k;
+};
+
+static int launch_stream(const StreamConfig& c, StreamArgs a, hipStream_t stream) {
+    const int frags = c.rg * c.mt;
+    a.waves = c.waves;
+    a.split_k = c.split_k;
+    a.n_tiles = (a.n + 16 * c.rg - 1) / (16 * c.rg);
+    a.m_tiles = (a.m + 16 * c.mt - 1) / (16 * c.mt);
+    const size_t lds = c.waves > 1 ? (size_t)c.waves * frags * 1024 : 0;
+    if (lds > 64 * 1024) return SG_INVALID_CONFIG;
+    const int total_stages = a.k / (c.ku * 64) > 0 ? a.k / (c.ku * 64) : 1;
+    if (c.split_k < 1 || c.split_k > total_stages) return SG_INVALID_CONFIG;
+    const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
+    if (tiles * c.split_k > 0x7fffffffu) return SG_BAD_ARGUMENT;
+    a.ws = nullptr;
+    a.counters = nullptr;
+    if (c.split_k > 1) {
+        Workspace* w;
+        if (int rc = get_workspace(&w)) return rc;
+        if (tiles > w->n_counters || tiles * c.split_k * frags * 1024 > w->partial_bytes) return SG_WORKSPACE_TOO_SMALL;
+        a.ws = w->partials;
+        a.counters = w->counters;
+    }
+    const unsigned grid = (unsigned)(tiles * c.split_k);
+    const unsigned threads = (unsigned)c.waves * 64;
+#define SG_GO(MT, RG) \
+    if (c.mt == MT && c.rg == RG) return SG_STREAM_LAUNCHER(MT, RG)(c.ku, c.depth, a, grid, threads, lds, stream);
+    SG_GO(1, 1) SG_GO(1, 2) SG_GO(1, 3) SG_GO(1, 4) SG_GO(2, 1) SG_GO(2, 2) SG_GO(2, 3) SG_GO(2, 4)
+#undef SG_GO
+    return SG_INVALID_CONFIG;
+}
+
+static int check_pointers(const void* A, const void* B, const void* D, int m, int n, int k, int b_stride) {
+    if (!A || !B || !D || m <= 0 || n <= 0 || k <= 0 || b_stride < k) return SG_BAD_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15u) return SG_BAD_ALIGNMENT;
+    if ((reinterpret_cast<uintptr_t>(D) & 7u) || (b_stride & 15)) return SG_BAD_ALIGNMENT;
+    return SG_SUCCESS;
+}
+
+// Shape -> configuration.  Weights are streamed once, so the only goals are (1) enough
+// workgroups and waves to cover every CU with tens of KB of loads in flight and (2) long
+// contiguous runs per weight row.  Numbers below come from sweeps on one MI355X.
+static StreamConfig pick_stream(int m, int n, int k, int cu_count) {
+    StreamConfig c;
+    c.mt = m <= 16 ? 1 : 2;
+    c.ku = (k % 256 == 0) ? 4 : ((k % 128 == 0) ? 2 : 1);
+    const int stages = (k + c.ku * 64 - 1) / (c.ku * 64);
+    c.rg = 1;
+    if ((n + 15) / 16 >= 8 * cu_count) c.rg = 2;
+    const int n_tiles = (n + 16 * c.rg - 1) / (16 * c.rg);
+    const int m_tiles = (m + 16 * c.mt - 1) / (16 * c.mt);
+    c.waves = stages >= 16 ? 8 : (stages >= 4 ? 4 : (stages >= 2 ? 2 : 1));
+    c.split_k = 1;
+    // few tiles: spread K over more workgroups until every CU has about two of them
+    while ((long)n_tiles * m_tiles * c.split_k < 2L * cu_count && stages / (c.split_k * 2) >= 2 * c.waves &&
+           c.split_k < 16)
+        c.split_k *= 2;
+    const int per_wave = stages / (c.split_k * c.waves);
+    c.depth = per_wave >= 4 ? 4 : (per_wave >= 2 ? 2 : 1);
+    while (stream_regs(c.mt, c.rg, c.ku, c.depth) > 128 && c.depth > 1) c.depth--;
+    if (c.depth == 3 && c.ku == 8) c.depth = 2;
+    return c;
+}
+
+}  // namespace sg
+
+using namespace sg;
+
+extern "C" {
+
+const char* sg_strerror(int code) {
+    switch (code) {
+        case SG_SUCCESS: return "success";
+        case SG_M_ABOVE_WARPTILE_M: return "m is greater than WARPTILE_M";
+        case SG_N_NOT_EVEN: return "n is not even";
+        case SG_K_NOT_DIVISIBLE_BY_WARPTILE_K: return "k is not divisible by WARPTILE_K";
+        case SG_TOO_MANY_WARPS: return "A_producers + B_producers + consumers is greater than 16";
+        case SG_QSIZE_TOO_SMALL: return "qsize is less than A_producers, B_producers / b_lanes, or consumers";
+        case SG_INVALID_CONFIG: return "no kernel is compiled for this configuration";
+        case SG_LAUNCH_FAILED: return "the HIP runtime refused the launch";
+        case SG_BAD_ALIGNMENT: return "pointer or stride is not sufficiently aligned";
+        case SG_BAD_ARGUMENT: return "null pointer or size out of range";
+        case SG_WORKSPACE_TOO_SMALL: return "split-K partials do not fit the workspace";
+        case SG_NO_DEVICE: return "no usable gfx950 device";
+        default: return "unknown code";
+    }
+}
+
+int sg_init(void) {
+    DeviceInfo* d;
+    if (int rc = get_device_info(&d)) return rc;
+    Workspace* w;
+    return get_workspace(&w);
+}
+
+size_t sg_workspace_bytes(void) { return kPartialBytes + kCounters * sizeof(unsigned); }
+
+int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,
+                   int b_stride, int split_k, int A_producers, int B_producers, int consumers, int b_lanes, int qsize,
+                   int op_m, int ops, void* stream) {
+    if (op_m != 8 && op_m != 16 && op_m != 32) return SG_INVALID_CONFIG;
+    if (ops <= 0 || b_lanes <= 0 || qsize <= 0 || split_k <= 0 || A_producers < 0 || B_producers < 0 || consumers <= 0)
+        return SG_INVALID_CONFIG;
+    const int warptile_k = (512 / op_m) * ops;
+    // same order as skinny_gemm/skinny_gemm_caller.cu:55-75
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % warptile_k != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (A_producers + B_producers + consumers > 16) return SG_TOO_MANY_WARPS;
+    const bool ring = A_producers > 0 || B_producers > 0;
+    if (ring && (qsize < A_producers || qsize < (B_producers / b_lanes) || qsize < consumers)) return SG_QSIZE_TOO_SMALL;
+    if (int rc = check_pointers(A, B, D, m, n, k, b_stride)) return rc;
+    if (!scale_tensor) return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+
+    if (ring) return SG_INVALID_CONFIG;  // LDS-ring variants are dispatched below once compiled in
+
+    if (warptile_k % 64 != 0) return SG_INVALID_CONFIG;
+    StreamConfig c;
+    c.mt = op_m == 32 ? 2 : 1;
+    c.rg = b_lanes;
+    c.ku = warptile_k / 64;
+    c.depth = qsize;
+    c.waves = consumers;
+    c.split_k = split_k;
+    StreamArgs a{};
+    a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
+    a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
+    a.out_f32 = 0;
+    return launch_stream(c, a, static_cast<hipStream_t>(stream));
+}
+
+int sg_skinny_gemm_pick(int m, int n, int k, int out[8]) {
+    if (!out || m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    int cu = 256;
+    if (get_device_info(&dev) == SG_SUCCESS) cu = dev->cu_count;
+    const StreamConfig c = pick_stream(m, n, k, cu);
+    const int op_m = c.mt == 2 ? 32 : (m <= 8 ? 8 : 16);
+    out[0] = c.split_k; out[1] = 0; out[2] = 0; out[3] = c.waves;
+    out[4] = c.rg; out[5] = c.depth; out[6] = op_m; out[7] = c.ku * 64 / (512 / op_m);
+    return SG_SUCCESS;
+}
+
+int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,
+                        int b_stride, void* stream) {
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 16 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (int rc = check_pointers(A, B, D, m, n, k, b_stride)) return rc;
+    if (!scale_tensor) return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    const StreamConfig c = pick_stream(m, n, k, dev->cu_count);
+    StreamArgs a{};
+    a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
+    a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
+    a.out_f32 = 0;
+    return launch_stream(c, a, static_cast<hipStream_t>(stream));
+}
+
+int sg_skinny_gemm_fastpath(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n,
+                            int k) {
+    return sg_skinny_gemm_auto(A, B, D, scale_tensor, m, n, k, k, nullptr);
+}
+
+static int async_gemm_common(const uint8_t* A, const uint8_t* B, void* D, int m, int n, int k, int out_f32) {
+    if (k % 64 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (int rc = check_pointers(A, B, D, m, n, k, k)) return rc;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    const StreamConfig c = pick_stream(m, n, k, dev->cu_count);
+    StreamArgs a{};
+    a.A = A; a.B = B; a.D = D; a.scale = nullptr;
+    a.m = m; a.n = n; a.k = k; a.b_stride = k;
+    a.out_f32 = out_f32;
+    return launch_stream(c, a, nullptr);
+}
+
+int sg_async_gemm_f32(const uint8_t* A, const uint8_t* B, float* D, int m, int n, int k) {
+    if (D && (reinterpret_cast<uintptr_t>(D) & 15u)) return SG_BAD_ALIGNMENT;
+    return async_gemm_common(A, B, D, m, n, k, 1);
+}
+
+int sg_async_gemm_bf16(const uint8_t* A, const uint8_t* B, void* D, int m, int n, int k) {
+    return async_gemm_common(A, B, D, m, n, k, 0);
+}
+
+int sg_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n, void* stream) {
+    return launch_tiled_sum_reduce(A, B, D, b, m, n, static_cast<hipStream_t>(stream));
+}
+
+int sg_fp8_encode_rows(const void* X, uint8_t* Q, float* scales, int rows, int cols, void* stream) {
+    return launch_fp8_encode_rows(X, Q, scales, rows, cols, static_cast<hipStream_t>(stream));
+}
+
+int sg_fp8_decode_rows(const uint8_t* Q, const float* scales, void* Y, int rows, int cols, void* stream) {
+    return launch_fp8_decode_rows(Q, scales, Y, rows, cols, static_cast<hipStream_t>(stream));
+}
+
+int sg_fp8_reduce_rows(const uint8_t* Q, const float* scales, void* Y, int nbuf, size_t q_buf_stride, int rows,
+                       int cols, void* stream) {
+    return launch_fp8_reduce_rows(Q, scales, Y, nbuf, q_buf_stride, rows, cols, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,42 @@
+// Device-side building blocks shared by the gfx950 kernels: vector types, bf16 rounding,
+// OCP E4M3 conversion helpers and cache-policy loads.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sg {
+
+typedef long  i64x2 __attribute__((ext_vector_type(2)));
+typedef int   i32x2 __attribute__((ext_vector_type(2)));
+typedef int   i32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
+
+// fp32 -> bf16 bits, round to nearest even; NaN stays a quiet NaN.
+__device__ __forceinline__ uint32_t bf16_bits(float x) {
+    uint32_t u = __float_as_uint(x);
+    uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return ((u & 0x7fffffffu) > 0x7f800000u) ? ((u >> 16) | 0x40u) : r;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return bf16_bits(lo) | (bf16_bits(hi) << 16);
+}
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// 16-byte global loads.  The streaming flavour marks the line non-temporal: weights are
+// read exactly once, so they should not displace the activations held in L2.
+__device__ __forceinline__ i64x2 load16(const void* p) { return *reinterpret_cast<const i64x2*>(p); }
+__device__ __forceinline__ i64x2 load16_stream(const void* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const i64x2*>(p));
+}
+
+}  // namespace sg

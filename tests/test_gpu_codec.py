@@ -1,0 +1,134 @@
+"""GPU parity of the per-row FP8 codec and the fp32 batch sum, through the C ABI.
+
+Encode must be byte-identical to the oracle.  Decode and reduce use the oracle's operation
+order (multiply and add rounded separately), so they are compared bit for bit as well; the
+tolerance named by the spec (1e-2) is asserted against an fp64 truth in addition.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import GEMM_TOL, bits, dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def sg():
+    import rocm_dev_amd
+    return rocm_dev_amd
+
+
+def _encode(sg, X):
+    rows, cols = X.shape
+    Xd = dev(X)
+    Q = torch.empty((rows, cols), dtype=torch.uint8, device="cuda")
+    S = torch.empty((rows,), dtype=torch.float32, device="cuda")
+    rc = sg.fp8_encode_rows(Xd, Q, S)
+    torch.cuda.synchronize()
+    assert rc == 0, sg.strerror(rc)
+    return Q, S
+
+
+@pytest.mark.parametrize("rows,cols", [(4, 16), (7, 512), (64, 1024), (33, 2064), (16, 8192), (5, 16384), (3, 40000 // 16 * 16)])
+def test_encode_bit_exact(sg, oracle, rows, cols):
+    X = oracle.normal_bf16_outliers((rows, cols), seed=rows, stream_id=3, frac=0.001, mag=50.0)
+    X[0] = 0                       # all-zero row -> scale 1, codes 0
+    X[-1, ::3] = 0x8000            # negative zeros keep their sign bit (code 0x80)
+    X[0, 1::2] = 0x8000
+    if rows > 2:
+        X[1] = (X[1].view(np.uint16) & 0x807F) | 0x0080   # tiny magnitudes (exponent 1): slow divide path
+        X[2] = 0x7F7F                                      # huge magnitudes
+    Q, S = _encode(sg, X)
+    q_ref, s_ref = oracle.fp8_encode_rows(X)
+    assert np.array_equal(S.cpu().numpy(), s_ref)
+    assert np.array_equal(Q.cpu().numpy(), q_ref)
+
+
+def test_encode_decode_reduce_config3_slice(sg, oracle):
+    """BASELINE config 3 recipe on a 512-row slice: 8 seeded buffers, outliers, encode, reduce."""
+    nbuf, rows, cols = 8, 512, 8192
+    Q = torch.empty((nbuf, rows, cols), dtype=torch.uint8, device="cuda")
+    S = torch.empty((nbuf, rows), dtype=torch.float32, device="cuda")
+    q_ref = np.empty((nbuf, rows, cols), np.uint8)
+    s_ref = np.empty((nbuf, rows), np.float32)
+    for i in range(nbuf):
+        X = oracle.normal_bf16_outliers((rows, cols), seed=i, stream_id=3, frac=0.001, mag=50.0)
+        assert sg.fp8_encode_rows(dev(X), Q[i], S[i]) == 0
+        q_ref[i], s_ref[i] = oracle.fp8_encode_rows(X)
+    torch.cuda.synchronize()
+    assert np.array_equal(Q.cpu().numpy(), q_ref)
+    assert np.array_equal(S.cpu().numpy(), s_ref)
+    # decode
+    Y = torch.empty((rows, cols), dtype=torch.bfloat16, device="cuda")
+    assert sg.fp8_decode_rows(Q[0], S[0], Y) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(Y), oracle.fp8_decode_rows(q_ref[0], s_ref[0]))
+    # reduce of 8
+    assert sg.fp8_reduce_rows(Q, S, Y) == 0
+    torch.cuda.synchronize()
+    got = bits(Y)
+    ref = oracle.fp8_reduce_rows(q_ref, s_ref)
+    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    assert np.array_equal(got, ref)
+    truth = sum(oracle.e4m3_decode(q_ref[i]).astype(np.float64) * s_ref[i].astype(np.float64)[:, None] for i in range(nbuf))
+    assert oracle.max_rel_err_bf16(got, oracle.bf16_from_f32(truth.astype(np.float32))) <= GEMM_TOL
+
+
+@pytest.mark.parametrize("nbuf", [1, 2, 3, 4, 5])
+def test_reduce_other_counts(sg, oracle, nbuf):
+    rows, cols = 40, 1040 // 16 * 16
+    q_ref = np.empty((nbuf, rows, cols), np.uint8)
+    s_ref = np.empty((nbuf, rows), np.float32)
+    for i in range(nbuf):
+        q_ref[i], s_ref[i] = oracle.fp8_encode_rows(oracle.normal_bf16_outliers((rows, cols), seed=10 + i, stream_id=3))
+    Y = torch.empty((rows, cols), dtype=torch.bfloat16, device="cuda")
+    assert sg.fp8_reduce_rows(dev(q_ref), dev(s_ref), Y) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(Y), oracle.fp8_reduce_rows(q_ref, s_ref))
+
+
+def test_full_size_properties(sg, oracle):
+    """8192 x 8192 (BASELINE config 3 size): properties that need no full-size oracle pass,
+    plus the oracle on the first and last 64 rows."""
+    rows = cols = 8192
+    g = torch.Generator(device="cuda").manual_seed(0)
+    X = torch.randn((rows, cols), generator=g, device="cuda", dtype=torch.float32).bfloat16()
+    idx = torch.randint(0, rows * cols, (67108,), generator=g, device="cuda")
+    X.view(-1)[idx] = torch.where(torch.rand(67108, generator=g, device="cuda") < 0.5, 50.0, -50.0).bfloat16()
+    Q = torch.empty((rows, cols), dtype=torch.uint8, device="cuda")
+    S = torch.empty((rows,), dtype=torch.float32, device="cuda")
+    assert sg.fp8_encode_rows(X, Q, S) == 0
+    Y = torch.empty((rows, cols), dtype=torch.bfloat16, device="cuda")
+    assert sg.fp8_decode_rows(Q, S, Y) == 0
+    torch.cuda.synchronize()
+    # scale is absmax/448 and the absmax element maps to +-448
+    amax = X.float().abs().amax(dim=1)
+    assert torch.equal(S.cpu(), amax.cpu() / 448.0)      # IEEE divide on the host
+    assert torch.all((Q & 0x7F).amax(dim=1) == 0x7E)
+    # decode(encode(x)) is within half an E4M3 step of x: |y - x| <= 2^-4 |x| + scale * 2^-10
+    err = (Y.float() - X.float()).abs()
+    bound = X.float().abs() * (2.0 ** -4 + 2.0 ** -8) + S[:, None] * 2.0 ** -9
+    assert torch.all(err <= bound)
+    # idempotence: encoding the decoded tensor reproduces the codes and the scales
+    Q2 = torch.empty_like(Q)
+    S2 = torch.empty_like(S)
+    assert sg.fp8_encode_rows(Y, Q2, S2) == 0
+    torch.cuda.synchronize()
+    same_rows = (S2 == S)
+    assert same_rows.float().mean() > 0.99
+    assert torch.equal(Q2[same_rows], Q[same_rows])
+    for sl in (slice(0, 64), slice(rows - 64, rows)):
+        q_ref, s_ref = oracle.fp8_encode_rows(bits(X[sl]))
+        assert np.array_equal(Q[sl].cpu().numpy(), q_ref)
+        assert np.array_equal(S[sl].cpu().numpy(), s_ref)
+
+
+@pytest.mark.parametrize("b,m,n", [(1, 8, 64), (5, 8, 64), (9, 24, 192), (3, 7, 33), (16, 128, 1024)])
+def test_tiled_sum_reduce(sg, oracle, b, m, n):
+    A = oracle.uniform_f32((b, m, n), 0, 7, -0.5, 0.5)
+    B = oracle.uniform_f32((b, m, n), 0, 8, -0.5, 0.5)
+    D = torch.empty((m, n), dtype=torch.float32, device="cuda")
+    assert sg.tiled_sum_reduce(dev(A), dev(B), D) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(D.cpu().numpy(), oracle.tiled_sum_reduce(A, B))
