@@ -97,6 +97,23 @@ int sg_skinny_gemm_fastpath(const uint8_t* A, const uint8_t* B, void* D_bf16, co
 int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
                         int m, int n, int k, int b_stride, void* stream);
 
+/* Library-native tuning record for sg_skinny_gemm_tuned - no counterpart in the reference,
+ * whose tunables are compile-time #defines rewritten by its grid-search script
+ * (grid.py:106-116); this is the run-time equivalent a tuning driver sweeps. */
+typedef struct SgTuning {
+    int engine;        /* 0 library's choice, 1 direct (global -> VGPR -> MFMA), 2 LDS ring (global -> LDS DMA -> MFMA) */
+    int split_k;       /* workgroups sharing one output tile along K */
+    int waves;         /* wavefronts per workgroup, sharing the tile along K (1..16) */
+    int row_tiles;     /* 16-row weight tiles per wavefront (b_lanes) */
+    int m_blocks;      /* 16-row activation blocks per tile: 1 (m <= 16 per tile) or 2 */
+    int depth;         /* stages in flight per wavefront (register ring / LDS ring slots) */
+    int k_chunks;      /* direct engine: 64-byte K chunks per stage (1, 2, 4, 8); LDS ring: fixed 256-byte stage */
+    int non_temporal;  /* LDS ring: stream weights with the non-temporal hint */
+} SgTuning;
+
+int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                         int m, int n, int k, int b_stride, const SgTuning* tuning, void* stream);
+
 /* The configuration sg_skinny_gemm_auto would use, for logging and tuning drivers.
  * out[8] = {split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops}. */
 int sg_skinny_gemm_pick(int m, int n, int k, int out[8]);

@@ -15,6 +15,7 @@ from .api import (  # noqa: F401
     skinny_gemm,
     skinny_gemm_fastpath,
     skinny_gemm_pick,
+    skinny_gemm_tuned,
     strerror,
     tiled_sum_reduce,
 )

@@ -11,6 +11,7 @@ reference's launchers do; ``check=True`` raises SgError instead.  Tensors are to
 tensors used purely as device buffers: fp8 operands are uint8 or float8_e4m3fn, outputs
 bfloat16 (or float32 for async_gemm), and everything is enqueued on torch's current stream.
 """
+import ctypes as C
 import enum
 
 import torch
@@ -88,9 +89,31 @@ def skinny_gemm_fastpath(A, B, D, scale_tensor, check=False):
     return _done(rc, check)
 
 
+class SgTuning(C.Structure):
+    """Mirror of the C struct SgTuning (include/sgemm.h)."""
+    _fields_ = [(name, C.c_int) for name in
+                ("engine", "split_k", "waves", "row_tiles", "m_blocks", "depth", "k_chunks", "non_temporal")]
+
+
+ENGINE_AUTO, ENGINE_DIRECT, ENGINE_LDS = 0, 1, 2
+
+
+def skinny_gemm_tuned(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k=1, waves=4, row_tiles=1, m_blocks=None,
+                      depth=2, k_chunks=4, non_temporal=1, check=False):
+    """The library-native tuning entry (no reference counterpart): pick the engine and its shape."""
+    m, k = A.shape
+    n = B.shape[0]
+    if m_blocks is None:
+        m_blocks = 1 if m <= 16 else 2
+    t = SgTuning(engine, split_k, waves, row_tiles, m_blocks, depth, k_chunks, non_temporal)
+    with torch.cuda.device(A.device):
+        rc = lib.sg_skinny_gemm_tuned(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
+                                      _dev(scale_tensor, torch.float32), m, n, k, B.stride(0), C.byref(t), _stream())
+    return _done(rc, check)
+
+
 def skinny_gemm_pick(m, n, k):
     """The tunables the fastpath would use: dict with the reference's parameter names."""
-    import ctypes as C
     out = (C.c_int * 8)()
     rc = lib.sg_skinny_gemm_pick(m, n, k, C.byref(out))
     if rc != 0:

@@ -1,9 +1,12 @@
 // C ABI of libsgemm.so: argument validation, configuration choice and launches.
 // The contract of every entry point is documented in include/sgemm.h.
+#include <cstdio>
+#include <cstdlib>
 #include <mutex>
 
 #include "sg_host.h"
 #include "sg_stream_kernel.h"
+#include <string>
 
 namespace sg {
 
@@ -22,6 +25,11 @@ static std::mutex g_mutex;
 static Workspace g_ws[kMaxDevices];
 static DeviceInfo g_dev[kMaxDevices];
 static bool g_dev_known[kMaxDevices];
+
+hipError_t report_hip(const char* what, hipError_t e) {
+    if (e != hipSuccess && getenv("SG_VERBOSE")) fprintf(stderr, "libsgemm: %s: %s\n", what, hipGetErrorString(e));
+    return e;
+}
 
 static int current_device(int* dev) {
     if (hipGetDevice(dev) != hipSuccess || *dev < 0 || *dev >= kMaxDevices) {
@@ -74,20 +82,28 @@ int get_workspace(Workspace** out) {
     return SG_SUCCESS;
 }
 
-// ---- streaming kernel dispatch ----------------------------------------------------------
-struct StreamConfig {
-    int mt, rg, ku, depth, waves, split_k;
+// ---- kernel dispatch ------------------------------------------------------------------------
+enum Engine { ENGINE_AUTO = 0, ENGINE_DIRECT = 1, ENGINE_LDS = 2, ENGINE_RING = 3 };
+
+struct Config {
+    int engine;   // ENGINE_DIRECT: global -> VGPR -> MFMA;  ENGINE_LDS: global -> LDS ring (DMA) -> MFMA
+    int mt;       // 16-row activation blocks per tile (1 or 2)
+    int rg;       // 16-row weight tiles per wave
+    int ku;       // direct engine: 64-byte K chunks per stage (the LDS engine's stage is 256 bytes)
+    int depth;    // stages in flight per wave
+    int waves;    // waves per workgroup, splitting K among themselves
+    int split_k;  // workgroups per tile, splitting K among themselves
+    int nt;       // weights loaded with the non-temporal hint
 };
 
-static int launch_stream(const StreamConfig& c, StreamArgs a, hipStream_t stream) {
+static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out) {
     const int frags = c.rg * c.mt;
+    if (c.waves < 1 || c.waves > 16 || c.depth < 1) return SG_INVALID_CONFIG;
     a.waves = c.waves;
     a.split_k = c.split_k;
     a.n_tiles = (a.n + 16 * c.rg - 1) / (16 * c.rg);
     a.m_tiles = (a.m + 16 * c.mt - 1) / (16 * c.mt);
-    const size_t lds = c.waves > 1 ? (size_t)c.waves * frags * 1024 : 0;
-    if (lds > 64 * 1024) return SG_INVALID_CONFIG;
-    const int total_stages = a.k / (c.ku * 64) > 0 ? a.k / (c.ku * 64) : 1;
+    const int total_stages = a.k / stage_bytes_k > 0 ? a.k / stage_bytes_k : 1;
     if (c.split_k < 1 || c.split_k > total_stages) return SG_INVALID_CONFIG;
     const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
     if (tiles * c.split_k > 0x7fffffffu) return SG_BAD_ARGUMENT;
@@ -100,12 +116,50 @@ static int launch_stream(const StreamConfig& c, StreamArgs a, hipStream_t stream
         a.ws = w->partials;
         a.counters = w->counters;
     }
+    *tiles_out = tiles;
+    return SG_SUCCESS;
+}
+
+static int launch_stream(const Config& c, StreamArgs a, hipStream_t stream) {
+    size_t tiles;
+    if (int rc = prepare(c, a, c.ku * 64, &tiles)) return rc;
+    const size_t lds = c.waves > 1 ? (size_t)c.waves * c.rg * c.mt * 1024 : 0;
+    if (lds > 64 * 1024) return SG_INVALID_CONFIG;
     const unsigned grid = (unsigned)(tiles * c.split_k);
     const unsigned threads = (unsigned)c.waves * 64;
 #define SG_GO(MT, RG) \
     if (c.mt == MT && c.rg == RG) return SG_STREAM_LAUNCHER(MT, RG)(c.ku, c.depth, a, grid, threads, lds, stream);
     SG_GO(1, 1) SG_GO(1, 2) SG_GO(1, 3) SG_GO(1, 4) SG_GO(2, 1) SG_GO(2, 2) SG_GO(2, 3) SG_GO(2, 4)
 #undef SG_GO
+    return SG_INVALID_CONFIG;
+}
+
+static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
+    if (a.k % 256 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    size_t tiles;
+    if (int rc = prepare(c, a, 256, &tiles)) return rc;
+    // activation DMA instructions per stage: 4 rows each, rounded up to a compiled count
+    int xu = 8;
+    if (c.mt == 1) {
+        const int need = (a.m + 3) / 4;
+        xu = need <= 1 ? 1 : (need <= 2 ? 2 : 4);
+    }
+    const size_t stage = (size_t)(c.rg * 4 + xu) * 1024;
+    // + 4 KB: lanes of activation rows that are not loaded read past the last slot
+    const size_t lds = (size_t)c.waves * c.depth * stage + 4096;
+    if (lds > 159 * 1024) return SG_INVALID_CONFIG;  // 160 KB per CU, minus the kernel's static LDS
+    const unsigned grid = (unsigned)(tiles * c.split_k);
+    const unsigned threads = (unsigned)c.waves * 64;
+#define SG_GO(MT, RG) \
+    if (c.mt == MT && c.rg == RG) return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, a, grid, threads, lds, stream);
+    SG_GO(1, 1) SG_GO(1, 2) SG_GO(1, 4) SG_GO(2, 1) SG_GO(2, 2) SG_GO(2, 4)
+#undef SG_GO
+    return SG_INVALID_CONFIG;
+}
+
+static int launch_config(const Config& c, const StreamArgs& a, hipStream_t stream) {
+    if (c.engine == ENGINE_DIRECT) return launch_stream(c, a, stream);
+    if (c.engine == ENGINE_LDS) return launch_lds(c, a, stream);
     return SG_INVALID_CONFIG;
 }
 
@@ -119,8 +173,10 @@ static int check_pointers(const void* A, const void* B, const void* D, int m, in
 // Shape -> configuration.  Weights are streamed once, so the only goals are (1) enough
 // workgroups and waves to cover every CU with tens of KB of loads in flight and (2) long
 // contiguous runs per weight row.  Numbers below come from sweeps on one MI355X.
-static StreamConfig pick_stream(int m, int n, int k, int cu_count) {
-    StreamConfig c;
+static Config pick_stream(int m, int n, int k, int cu_count) {
+    Config c;
+    c.engine = ENGINE_DIRECT;
+    c.nt = 1;
     c.mt = m <= 16 ? 1 : 2;
     c.ku = (k % 256 == 0) ? 4 : ((k % 128 == 0) ? 2 : 1);
     const int stages = (k + c.ku * 64 - 1) / (c.ku * 64);
@@ -131,7 +187,7 @@ static StreamConfig pick_stream(int m, int n, int k, int cu_count) {
     c.waves = stages >= 16 ? 8 : (stages >= 4 ? 4 : (stages >= 2 ? 2 : 1));
     c.split_k = 1;
     // few tiles: spread K over more workgroups until every CU has about two of them
-    while ((long)n_tiles * m_tiles * c.split_k < 2L * cu_count && stages / (c.split_k * 2) >= 2 * c.waves &&
+    while ((long)n_tiles * m_tiles * c.split_k < cu_count / 2 && stages / (c.split_k * 2) >= 2 * c.waves &&
            c.split_k < 16)
         c.split_k *= 2;
     const int per_wave = stages / (c.split_k * c.waves);
@@ -192,21 +248,57 @@ int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* sca
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
 
-    if (ring) return SG_INVALID_CONFIG;  // LDS-ring variants are dispatched below once compiled in
+    if (ring) return SG_INVALID_CONFIG;  // producer/consumer ring variants are dispatched here once compiled in
 
     if (warptile_k % 64 != 0) return SG_INVALID_CONFIG;
-    StreamConfig c;
+    Config c;
     c.mt = op_m == 32 ? 2 : 1;
     c.rg = b_lanes;
     c.ku = warptile_k / 64;
     c.depth = qsize;
     c.waves = consumers;
     c.split_k = split_k;
+    c.nt = 1;
+    // a 256-byte stage with at least two ring slots is the LDS ring's shape; everything else
+    // streams straight into registers
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
     a.out_f32 = 0;
-    return launch_stream(c, a, static_cast<hipStream_t>(stream));
+    if (warptile_k == 256 && qsize >= 2 && k % 256 == 0 && (b_lanes == 1 || b_lanes == 2 || b_lanes == 4)) {
+        c.engine = ENGINE_LDS;
+        const int rc = launch_config(c, a, static_cast<hipStream_t>(stream));
+        if (rc != SG_INVALID_CONFIG) return rc;   // ring does not fit LDS: stream through registers instead
+    }
+    c.engine = ENGINE_DIRECT;
+    return launch_config(c, a, static_cast<hipStream_t>(stream));
+}
+
+int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,
+                         int b_stride, const SgTuning* t, void* stream) {
+    if (!t) return SG_BAD_ARGUMENT;
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 16 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (int rc = check_pointers(A, B, D, m, n, k, b_stride)) return rc;
+    if (!scale_tensor) return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    Config c;
+    c.engine = t->engine;
+    c.mt = t->m_blocks;
+    c.rg = t->row_tiles;
+    c.ku = t->k_chunks;
+    c.depth = t->depth;
+    c.waves = t->waves;
+    c.split_k = t->split_k;
+    c.nt = t->non_temporal;
+    if (c.engine == ENGINE_AUTO) c = pick_stream(m, n, k, dev->cu_count);
+    if (c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
+    StreamArgs a{};
+    a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
+    a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
+    a.out_f32 = 0;
+    return launch_config(c, a, static_cast<hipStream_t>(stream));
 }
 
 int sg_skinny_gemm_pick(int m, int n, int k, int out[8]) {
@@ -214,7 +306,7 @@ int sg_skinny_gemm_pick(int m, int n, int k, int out[8]) {
     DeviceInfo* dev;
     int cu = 256;
     if (get_device_info(&dev) == SG_SUCCESS) cu = dev->cu_count;
-    const StreamConfig c = pick_stream(m, n, k, cu);
+    const Config c = pick_stream(m, n, k, cu);
     const int op_m = c.mt == 2 ? 32 : (m <= 8 ? 8 : 16);
     out[0] = c.split_k; out[1] = 0; out[2] = 0; out[3] = c.waves;
     out[4] = c.rg; out[5] = c.depth; out[6] = op_m; out[7] = c.ku * 64 / (512 / op_m);
@@ -229,12 +321,12 @@ int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D, const float
     if (!scale_tensor) return SG_BAD_ARGUMENT;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const StreamConfig c = pick_stream(m, n, k, dev->cu_count);
+    const Config c = pick_stream(m, n, k, dev->cu_count);
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
     a.out_f32 = 0;
-    return launch_stream(c, a, static_cast<hipStream_t>(stream));
+    return launch_config(c, a, static_cast<hipStream_t>(stream));
 }
 
 int sg_skinny_gemm_fastpath(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n,
@@ -247,12 +339,12 @@ static int async_gemm_common(const uint8_t* A, const uint8_t* B, void* D, int m,
     if (int rc = check_pointers(A, B, D, m, n, k, k)) return rc;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const StreamConfig c = pick_stream(m, n, k, dev->cu_count);
+    const Config c = pick_stream(m, n, k, dev->cu_count);
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = nullptr;
     a.m = m; a.n = n; a.k = k; a.b_stride = k;
     a.out_f32 = out_f32;
-    return launch_stream(c, a, nullptr);
+    return launch_config(c, a, nullptr);
 }
 
 int sg_async_gemm_f32(const uint8_t* A, const uint8_t* B, float* D, int m, int n, int k) {

@@ -1,0 +1,131 @@
+// Arguments and epilogue shared by the dense GEMM kernels: cross-wave reduction through LDS,
+// cross-workgroup split-K through the fp32 workspace, scale, bf16 rounding and the store.
+//
+// Fragment convention (both kernels): acc[rg][mt] is the 16 x 16 fp32 tile of weight rows
+// n0 + 16*rg .. +15 against activation rows m0 + 16*mt .. +15 in the MFMA result layout:
+// lane l owns activation row (l % 16) and weight rows 4*(l / 16) .. +3, i.e. four
+// consecutive n of one output row.
+//
+// Reference behaviour restated: every partial of every consumer wave and of every K split
+// is added into D (skinny_gemm/consumers/mfma_16x16x32_consumer.cu:119-162 does it with
+// fp16 atomics into a pre-zeroed D).  Here the partials are summed in fp32 in a fixed
+// order - waves in wave order through LDS, K splits in split order through the workspace
+// by the last workgroup to arrive - then scaled and rounded to bf16 once, and D is
+// overwritten.
+#pragma once
+
+#include "sg_device.h"
+
+namespace sg {
+
+struct StreamArgs {
+    const uint8_t* A;
+    const uint8_t* B;
+    void* D;                // bf16 or fp32, [m, n]
+    const float* scale;     // device scalar, or nullptr for 1.0f
+    float* ws;              // split-K partials (fp32)
+    unsigned* counters;     // one arrival counter per output tile, zero between launches
+    int m, n, k, b_stride;
+    int split_k, waves;
+    int n_tiles, m_tiles;
+    int out_f32;
+};
+
+// Writes one finished 16(n) x 16(m) fragment: lane owns m = m_base + l%16, n = n_base + 4*(l/16)..+3.
+__device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, float scale, int m_idx, int n_idx) {
+    if (m_idx >= a.m) return;
+    v *= scale;
+    const size_t off = (size_t)m_idx * a.n + n_idx;
+    if (a.out_f32) {
+        float* d = reinterpret_cast<float*>(a.D) + off;
+        if (n_idx + 3 < a.n && (a.n & 3) == 0) {
+            *reinterpret_cast<f32x4*>(d) = v;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (n_idx + e < a.n) d[e] = v[e];
+        }
+    } else {
+        uint16_t* d = reinterpret_cast<uint16_t*>(a.D) + off;
+        if (n_idx + 3 < a.n && (a.n & 3) == 0) {
+            u32x2 p = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+            *reinterpret_cast<u32x2*>(d) = p;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (n_idx + e < a.n) d[e] = (uint16_t)bf16_bits(v[e]);
+        }
+    }
+}
+
+template <int RG, int MT>
+__device__ __forceinline__ void finish_tile(const StreamArgs& a, f32x4 (&acc)[RG][MT], f32x4* red, unsigned* arrival_lds,
+                                            int tile_m, int tile_n, int split, int m0, int n0) {
+    constexpr int FRAGS = RG * MT;
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int waves = a.waves;
+    const int r = lane & 15, g = lane >> 4;
+    unsigned& arrival = *arrival_lds;
+    const float scale = a.scale ? a.scale[0] : 1.0f;
+    const int tile_id = tile_m * a.n_tiles + tile_n;
+    float* ws_tile = a.ws + ((size_t)tile_id * a.split_k) * (FRAGS * 256);
+
+    auto finish = [&](int f, f32x4 v) {
+        const int rg = f / MT, mt = f % MT;
+        if (a.split_k == 1) {
+            store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g);
+        } else {
+            // agent-scope stores go through to memory, past this XCD's L2, so that a workgroup on
+            // another XCD can read them without any cache-wide write-back or invalidate
+            float* p = ws_tile + ((size_t)split * FRAGS + f) * 256 + lane;
+#pragma unroll
+            for (int e = 0; e < 4; e++) __hip_atomic_store(p + e * 64, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    };
+
+    if (waves == 1) {
+#pragma unroll
+        for (int f = 0; f < FRAGS; f++) finish(f, acc[f / MT][f % MT]);
+    } else {
+#pragma unroll
+        for (int f = 0; f < FRAGS; f++) red[(f * waves + wave) * 64 + lane] = acc[f / MT][f % MT];
+        __syncthreads();
+        for (int f = wave; f < FRAGS; f += waves) {
+            f32x4 v = red[(f * waves) * 64 + lane];
+            for (int w = 1; w < waves; w++) v += red[(f * waves + w) * 64 + lane];
+            finish(f, v);
+        }
+    }
+
+    if (a.split_k == 1) return;
+
+    // ---- cross-workgroup split-K: last arrival sums the partials in split order --------
+    // Order without cache-wide fences: the partial stores above are agent-scope (write-through);
+    // each wave waits until its stores are acknowledged, the workgroup barrier collects all
+    // waves, then one thread bumps the tile's arrival counter.  The workgroup that observes
+    // split_k - 1 earlier arrivals reads every partial with agent-scope loads.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0)
+        arrival = __hip_atomic_fetch_add(&a.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (arrival != (unsigned)(a.split_k - 1)) return;
+    for (int f = wave; f < FRAGS; f += waves) {
+        const float* p = ws_tile + (size_t)f * 256 + lane;
+        f32x4 v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = __hip_atomic_load(p + e * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int sp = 1; sp < a.split_k; sp++) {
+            const float* q = p + (size_t)sp * FRAGS * 256;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] += __hip_atomic_load(q + e * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        const int rg = f / MT, mt = f % MT;
+        store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g);
+    }
+    if (threadIdx.x == 0)  // ready for the next launch
+        __hip_atomic_store(&a.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace sg

@@ -21,6 +21,17 @@ struct StreamArgs;
 SG_DECL_STREAM(1, 1) SG_DECL_STREAM(1, 2) SG_DECL_STREAM(1, 3) SG_DECL_STREAM(1, 4)
 SG_DECL_STREAM(2, 1) SG_DECL_STREAM(2, 2) SG_DECL_STREAM(2, 3) SG_DECL_STREAM(2, 4)
 
+#define SG_CAT_LDS_(a, b, c) a##b##_##c
+#define SG_CAT_LDS(a, b, c) SG_CAT_LDS_(a, b, c)
+#define SG_LDS_LAUNCHER(MT, RG) SG_CAT_LDS(launch_lds_, MT, RG)
+#define SG_DECL_LDS(MT, RG)                                                                              \
+    int SG_LDS_LAUNCHER(MT, RG)(int xu, int depth, int nt, const StreamArgs& a, unsigned grid, unsigned threads, \
+                                size_t lds, hipStream_t stream);
+SG_DECL_LDS(1, 1) SG_DECL_LDS(1, 2) SG_DECL_LDS(1, 4) SG_DECL_LDS(2, 1) SG_DECL_LDS(2, 2) SG_DECL_LDS(2, 4)
+
+// Prints a HIP failure to stderr when the environment variable SG_VERBOSE is set; returns e.
+hipError_t report_hip(const char* what, hipError_t e);
+
 // Split-K workspace of the current device (created on first use).
 struct Workspace {
     float* partials = nullptr;

@@ -1,0 +1,57 @@
+// One translation unit per (SG_MT, SG_RG): instantiates the LDS-ring kernel for every
+// compiled (XU, DEPTH, NT) and exposes a launcher the dispatcher in sg_api.hip calls.
+#include "sg_lds_kernel.h"
+#include "sg_host.h"
+
+#ifndef SG_MT
+#error "compile with -DSG_MT=<1|2> -DSG_RG=<1|2|4>"
+#endif
+
+namespace sg {
+
+template <int XU, int DEPTH, bool NT>
+static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
+    auto kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
+    // dynamic LDS above the default cap must be requested per kernel; remember the largest
+    // request made so far on each device
+    static size_t attr_bytes[16] = {};
+    if (lds > 48 * 1024) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
+        if (attr_bytes[dev] < lds) {
+            if (report_hip("hipFuncSetAttribute",
+                           hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
+                (void)hipGetLastError();
+                return SG_LAUNCH_FAILED;
+            }
+            attr_bytes[dev] = lds;
+        }
+    }
+    kernel<<<dim3(grid), dim3(threads), lds, stream>>>(a);
+    return report_hip("lds_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
+}
+
+#define SG_CASE(XU_, DEPTH_)                                                                    \
+    if (xu == XU_ && depth == DEPTH_) {                                                         \
+        if constexpr ((DEPTH_ - 1) * (SG_RG * 4 + XU_) <= 63 && XU_ <= 4 * SG_MT) {             \
+            return nt ? launch_one<XU_, DEPTH_, true>(a, grid, threads, lds, stream)            \
+                      : launch_one<XU_, DEPTH_, false>(a, grid, threads, lds, stream);          \
+        } else {                                                                                \
+            return SG_INVALID_CONFIG;                                                           \
+        }                                                                                       \
+    }
+
+int SG_LDS_LAUNCHER(SG_MT, SG_RG)(int xu, int depth, int nt, const StreamArgs& a, unsigned grid, unsigned threads,
+                                  size_t lds, hipStream_t stream) {
+#if SG_MT == 1
+    SG_CASE(1, 2) SG_CASE(1, 3) SG_CASE(1, 4) SG_CASE(1, 6) SG_CASE(1, 8)
+    SG_CASE(2, 2) SG_CASE(2, 3) SG_CASE(2, 4) SG_CASE(2, 6) SG_CASE(2, 8)
+    SG_CASE(4, 2) SG_CASE(4, 3) SG_CASE(4, 4) SG_CASE(4, 6) SG_CASE(4, 8)
+#else
+    SG_CASE(8, 2) SG_CASE(8, 3) SG_CASE(8, 4) SG_CASE(8, 6) SG_CASE(8, 8)
+#endif
+    return SG_INVALID_CONFIG;
+}
+
+}  // namespace sg

@@ -1,0 +1,189 @@
+// LDS-ring FP8 skinny GEMM for gfx950:  D[m,n] = scale * sum_k A[m,k] * B[n,k].
+//
+// Why LDS.  HBM3E wants long contiguous runs: a wave instruction that reads 4 rows x 256
+// contiguous bytes sustains about 15 % more bandwidth than one that reads 16 rows x 64
+// bytes (what the MFMA register layout would ask for).  So both operands are fetched with
+// the wide pattern by gfx950's direct-to-LDS loads (global_load_lds_dwordx4: no VGPR
+// staging, tracked by vmcnt) into a ring of stages, and read back from LDS in the MFMA
+// layout.
+//
+// One stage = 256 bytes of K ("K block") for the 16*RG weight rows and the activation rows
+// of the tile.  One DMA instruction moves 4 rows x 256 B = 1 KB; the hardware puts lane l's
+// 16 bytes at  ring slot base + 16*l.  Which global chunk a lane fetches is ours to choose,
+// and a permutation inside each 64-byte run costs nothing in the memory system, so
+// instruction u (rows 4u..4u+3 of a 16-row group) lets lane l = 4*q + p fetch
+//     row 4u + (q % 4),  K bytes  64*(q / 4) + 16*((p + u) % 4) .. +15,
+// i.e. it rotates the four 16-byte pieces of every 64-byte run by u.  The MFMA read of
+// lane (r = l%16, g = l/16) for 64-byte chunk kc is then the 16 bytes at
+//     1024*(r/4) + 64*(4*kc + r%4) + 16*((g - r/4) & 3),
+// and the sixteen lanes of one ds_read_b128 pass (same g, r = 0..15) hit sixteen different
+// 4-bank groups: no bank conflicts, no padding.
+//
+// Ring protocol.  Every wave is producer and consumer of its own ring: it issues the DMAs
+// of DEPTH stages ahead, waits with s_waitcnt vmcnt(n) until the oldest stage has landed
+// (loads complete in order), consumes it, and refills the slot.  Nothing but the wave's own
+// counters is involved, so there are no flags to poll and no barrier until the epilogue.
+// (The variant with separate producer and consumer waves is sg_ring_kernel.h.)
+//
+// The DMA is issued from inline assembly so that the compiler's wait-count insertion does
+// not see it: it would otherwise wait for ALL outstanding DMAs before every LDS read.
+#pragma once
+
+#include "sg_device.h"
+#include "sg_epilogue.h"
+
+namespace sg {
+
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+    return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+// 64 lanes x 16 bytes from global memory to LDS [lds_base + 16*lane]; lds_base is wave-uniform.
+__device__ __forceinline__ void dma_1kb(const void* gptr, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_base) : "memory");
+}
+__device__ __forceinline__ void dma_1kb_stream(const void* gptr, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Drains the last DEPTH stages: stage D of them still has DEPTH-1-D younger stages in flight.
+template <int D, int DEPTH, int PER_STAGE, class Consume>
+__device__ __forceinline__ void drain_ring(Consume& consume, int i) {
+    wait_vmcnt<(DEPTH - 1 - D) * PER_STAGE>();
+    consume(i + D);
+    if constexpr (D + 1 < DEPTH) drain_ring<D + 1, DEPTH, PER_STAGE>(consume, i);
+}
+
+constexpr int lds_stage_bytes(int RG, int XU) { return (RG * 4 + XU) * 1024; }
+
+// XU = activation DMA instructions per stage (4 rows each): ceil(min(m, 16*MT) / 4)
+template <int MT, int RG, int XU, int DEPTH, bool NT>
+__global__ void __launch_bounds__(1024) lds_gemm_kernel(const StreamArgs a) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
+    __shared__ unsigned arrival;
+
+    constexpr int PER_STAGE = RG * 4 + XU;         // DMA instructions per stage
+    constexpr int STAGE_BYTES = PER_STAGE * 1024;
+    static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
+    static_assert(XU <= 4 * MT, "more activation rows than the tile has");
+
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int waves = a.waves;
+
+    int bid = blockIdx.x;
+    const int tile_n = bid % a.n_tiles;
+    bid /= a.n_tiles;
+    const int split = bid % a.split_k;
+    const int tile_m = bid / a.split_k;
+    const int n0 = tile_n * (16 * RG);
+    const int m0 = tile_m * (16 * MT);
+
+    // K range of this workgroup in 256-byte blocks; the last split takes the remainder
+    const int blocks = a.k >> 8;
+    const int per_split = blocks / a.split_k;
+    const int b_begin = split * per_split;
+    const int b_end = (split == a.split_k - 1) ? blocks : b_begin + per_split;
+    const int n_blk = b_end - b_begin;
+    const int mine = wave < n_blk ? (n_blk - wave + waves - 1) / waves : 0;
+
+    // ---- DMA source pointers (per lane) ---------------------------------------------------
+    const int q = lane >> 2, p = lane & 3;
+    const int src_row = q & 3;        // row inside the 4-row instruction
+    const int src_kc = q >> 2;        // 64-byte run inside the 256-byte block
+    const uint8_t* wsrc[RG][4];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            int row = n0 + rg * 16 + 4 * u + src_row;
+            row = row < a.n ? row : a.n - 1;   // past the edge: re-read the last row, never stored
+            wsrc[rg][u] = a.B + (size_t)row * a.b_stride + src_kc * 64 + ((p + u) & 3) * 16;
+        }
+    const uint8_t* xsrc[XU];
+#pragma unroll
+    for (int u = 0; u < XU; u++) {
+        int row = m0 + 4 * u + src_row;
+        row = row < a.m ? row : a.m - 1;
+        xsrc[u] = a.A + (size_t)row * a.k + src_kc * 64 + ((p + (u & 3)) & 3) * 16;
+    }
+
+    // ---- LDS read offsets (per lane) ------------------------------------------------------
+    const int r = lane & 15, g = lane >> 4;
+    const int rd_off = 1024 * (r >> 2) + 64 * (r & 3) + 16 * ((g - (r >> 2)) & 3);
+    const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
+    const unsigned my_ring_lds = lds_addr(my_ring);
+
+    auto issue = [&](int i) {  // i-th stage of this wave -> slot i % DEPTH
+        const size_t koff = (size_t)(b_begin + wave + i * waves) << 8;
+        const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (NT) dma_1kb_stream(wsrc[rg][u] + koff, slot + (rg * 4 + u) * 1024);
+                else dma_1kb(wsrc[rg][u] + koff, slot + (rg * 4 + u) * 1024);
+            }
+#pragma unroll
+        for (int u = 0; u < XU; u++) dma_1kb(xsrc[u] + koff, slot + (RG * 4 + u) * 1024);
+    };
+
+    f32x4 acc[RG][MT];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto consume = [&](int i) {
+        const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
+#pragma unroll
+        for (int kc = 0; kc < 4; kc++) {
+            i64x2 x[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+                x[mt] = *reinterpret_cast<const i64x2*>(slot + (RG * 4 + mt * 4) * 1024 + kc * 256);
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                const i64x2 w = *reinterpret_cast<const i64x2*>(slot + rg * 4096 + kc * 256);
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.x, x[mt].x, acc[rg][mt], 0, 0, 0);
+                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.y, x[mt].y, acc[rg][mt], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    if (mine >= DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) issue(d);
+        int i = 0;
+        for (; i + DEPTH < mine; i++) {
+            wait_vmcnt<(DEPTH - 1) * PER_STAGE>();   // stage i has landed; DEPTH-1 stages still in flight
+            consume(i);
+            // the slot is refilled only after its reads have returned: the MFMAs above need the
+            // data, and this wait keeps the DMA behind them
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            issue(i + DEPTH);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        drain_ring<0, DEPTH, PER_STAGE>(consume, i);
+    } else {
+        for (int i = 0; i < mine; i++) issue(i);
+        wait_vmcnt<0>();
+        for (int i = 0; i < mine; i++) consume(i);
+    }
+
+    // the ring is reused for the cross-wave reduction: every wave must be done reading it
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    finish_tile<RG, MT>(a, acc, reinterpret_cast<f32x4*>(ring), &arrival, tile_m, tile_n, split, m0, n0);
+}
+
+}  // namespace sg

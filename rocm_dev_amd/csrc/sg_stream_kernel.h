@@ -28,21 +28,9 @@
 #pragma once
 
 #include "sg_device.h"
+#include "sg_epilogue.h"
 
 namespace sg {
-
-struct StreamArgs {
-    const uint8_t* A;
-    const uint8_t* B;
-    void* D;                // bf16 or fp32, [m, n]
-    const float* scale;     // device scalar, or nullptr for 1.0f
-    float* ws;              // split-K partials (fp32)
-    unsigned* counters;     // one arrival counter per output tile, zero between launches
-    int m, n, k, b_stride;
-    int split_k, waves;
-    int n_tiles, m_tiles;
-    int out_f32;
-};
 
 constexpr int stream_regs(int MT, int RG, int KU, int DEPTH) {
     return DEPTH * KU * (RG + MT) * 4 + RG * MT * 4 + 28;
@@ -88,33 +76,6 @@ __device__ __forceinline__ void mma_stage(const Stage<MT, RG, KU>& st, f32x4 (&a
                 acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(st.w[rg][u].x, st.x[mt][u].x, acc[rg][mt], 0, 0, 0);
                 acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(st.w[rg][u].y, st.x[mt][u].y, acc[rg][mt], 0, 0, 0);
             }
-        }
-    }
-}
-
-// Writes one finished 16(n) x 16(m) fragment: lane owns m = m_base + l%16, n = n_base + 4*(l/16)..+3.
-__device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, float scale, int m_idx, int n_idx) {
-    if (m_idx >= a.m) return;
-    v *= scale;
-    const size_t off = (size_t)m_idx * a.n + n_idx;
-    if (a.out_f32) {
-        float* d = reinterpret_cast<float*>(a.D) + off;
-        if (n_idx + 3 < a.n && (a.n & 3) == 0) {
-            *reinterpret_cast<f32x4*>(d) = v;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (n_idx + e < a.n) d[e] = v[e];
-        }
-    } else {
-        uint16_t* d = reinterpret_cast<uint16_t*>(a.D) + off;
-        if (n_idx + 3 < a.n && (a.n & 3) == 0) {
-            u32x2 p = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-            *reinterpret_cast<u32x2*>(d) = p;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                if (n_idx + e < a.n) d[e] = (uint16_t)bf16_bits(v[e]);
         }
     }
 }
@@ -223,51 +184,7 @@ stream_gemm_kernel(const StreamArgs a) {
         mma_stage<MT, RG, KU>(st[0], acc);
     }
 
-    // ---- reduce the waves' partial tiles through LDS, in wave order -------------------
-    const float scale = a.scale ? a.scale[0] : 1.0f;
-    const int tile_id = tile_m * a.n_tiles + tile_n;
-    float* ws_tile = a.ws + ((size_t)tile_id * a.split_k) * (FRAGS * 256);
-
-    auto finish = [&](int f, f32x4 v) {
-        const int rg = f / MT, mt = f % MT;
-        if (a.split_k == 1) {
-            store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g);
-        } else {
-            reinterpret_cast<f32x4*>(ws_tile + ((size_t)split * FRAGS + f) * 256)[lane] = v;
-        }
-    };
-
-    if (waves == 1) {
-#pragma unroll
-        for (int f = 0; f < FRAGS; f++) finish(f, acc[f / MT][f % MT]);
-    } else {
-#pragma unroll
-        for (int f = 0; f < FRAGS; f++) red[(f * waves + wave) * 64 + lane] = acc[f / MT][f % MT];
-        __syncthreads();
-        for (int f = wave; f < FRAGS; f += waves) {
-            f32x4 v = red[(f * waves) * 64 + lane];
-            for (int w = 1; w < waves; w++) v += red[(f * waves + w) * 64 + lane];
-            finish(f, v);
-        }
-    }
-
-    if (a.split_k == 1) return;
-
-    // ---- cross-workgroup split-K: last arrival sums the partials in split order --------
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) arrival = atomicAdd(&a.counters[tile_id], 1u);
-    __syncthreads();
-    if (arrival != (unsigned)(a.split_k - 1)) return;
-    __threadfence();
-    for (int f = wave; f < FRAGS; f += waves) {
-        const f32x4* p = reinterpret_cast<const f32x4*>(ws_tile + (size_t)f * 256) + lane;
-        f32x4 v = __builtin_nontemporal_load(p);
-        for (int sp = 1; sp < a.split_k; sp++) v += __builtin_nontemporal_load(p + (size_t)sp * FRAGS * 64);
-        const int rg = f / MT, mt = f % MT;
-        store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g);
-    }
-    if (threadIdx.x == 0) a.counters[tile_id] = 0;  // ready for the next launch
+    finish_tile<RG, MT>(a, acc, red, &arrival, tile_m, tile_n, split, m0, n0);
 }
 
 }  // namespace sg

@@ -112,6 +112,47 @@ def test_explicit_configs(sg, oracle, cfg, shape):
     assert np.array_equal(bits(D2), got)
 
 
+LDS_CONFIGS = [
+    # split_k, waves, row_tiles, depth, non_temporal
+    (1, 1, 1, 2, 1),
+    (1, 4, 1, 4, 1),
+    (1, 8, 1, 2, 0),
+    (1, 4, 2, 3, 1),
+    (1, 2, 4, 2, 1),
+    (2, 4, 1, 4, 1),
+    (4, 2, 2, 2, 0),
+    (1, 3, 1, 6, 1),
+    (1, 2, 1, 8, 1),
+    (1, 16, 1, 2, 1),
+]
+
+
+@pytest.mark.parametrize("cfg", LDS_CONFIGS)
+@pytest.mark.parametrize("shape", [(1, 256, 2048), (4, 96, 1024), (8, 512, 4096), (13, 130, 3072), (16, 1024, 1024),
+                                   (32, 512, 2048), (27, 100, 1280), (40, 64, 512)])
+def test_lds_ring_engine(sg, oracle, cfg, shape):
+    """The direct-to-LDS ring engine (global_load_lds DMA, conflict-free MFMA reads)."""
+    split_k, waves, row_tiles, depth, nt = cfg
+    m, n, k = shape
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=6)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = sg.skinny_gemm_tuned(A, B, D, S, engine=2, split_k=split_k, waves=waves, row_tiles=row_tiles, depth=depth,
+                              non_temporal=nt)
+    torch.cuda.synchronize()
+    if rc == 6:
+        pytest.skip("configuration not compiled / does not fit LDS")
+    assert rc == 0, sg.strerror(rc)
+    got = bits(D)
+    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_tuned(A, B, D2, S, engine=2, split_k=split_k, waves=waves, row_tiles=row_tiles, depth=depth,
+                                non_temporal=nt) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(D2), got)
+
+
 def test_torch_binding_surface(sg, oracle):
     """HFRK_skinny_gemm as the reference's Python callers use it: B passed as a (k, n) view."""
     m, n, k = 8, 1024, 2048
