@@ -109,6 +109,7 @@ typedef struct SgTuning {
     int depth;         /* stages in flight per wavefront (register ring / LDS ring slots) */
     int k_chunks;      /* direct engine: 64-byte K chunks per stage (1, 2, 4, 8); LDS ring: fixed 256-byte stage */
     int non_temporal;  /* LDS ring: stream weights with the non-temporal hint */
+    int persistent_wgs_per_cu; /* LDS ring: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU */
 } SgTuning;
 
 int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,

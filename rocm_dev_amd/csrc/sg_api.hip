@@ -94,6 +94,7 @@ struct Config {
     int waves;    // waves per workgroup, splitting K among themselves
     int split_k;  // workgroups per tile, splitting K among themselves
     int nt;       // weights loaded with the non-temporal hint
+    int persist;  // LDS engine: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU walking the tiles
 };
 
 static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out) {
@@ -146,12 +147,21 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     }
     const size_t stage = (size_t)(c.rg * 4 + xu) * 1024;
     // + 4 KB: lanes of activation rows that are not loaded read past the last slot
-    const size_t lds = (size_t)c.waves * c.depth * stage + 4096;
+    size_t lds = (size_t)c.waves * c.depth * stage + 4096;
+    unsigned grid = (unsigned)(tiles * c.split_k);
+    if (c.persist > 0) {
+        if (c.split_k != 1) return SG_INVALID_CONFIG;
+        lds += 2u * c.waves * c.rg * c.mt * 1024;   // double-buffered reduction scratch
+        DeviceInfo* dev;
+        if (int rc = get_device_info(&dev)) return rc;
+        const size_t want = (size_t)dev->cu_count * c.persist;
+        if (want < grid) grid = (unsigned)want;
+    }
     if (lds > 159 * 1024) return SG_INVALID_CONFIG;  // 160 KB per CU, minus the kernel's static LDS
-    const unsigned grid = (unsigned)(tiles * c.split_k);
     const unsigned threads = (unsigned)c.waves * 64;
-#define SG_GO(MT, RG) \
-    if (c.mt == MT && c.rg == RG) return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, a, grid, threads, lds, stream);
+#define SG_GO(MT, RG)                                                                                          \
+    if (c.mt == MT && c.rg == RG)                                                                              \
+        return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, c.persist > 0, a, grid, threads, lds, stream);
     SG_GO(1, 1) SG_GO(1, 2) SG_GO(1, 4) SG_GO(2, 1) SG_GO(2, 2) SG_GO(2, 4)
 #undef SG_GO
     return SG_INVALID_CONFIG;
@@ -171,22 +181,51 @@ static int check_pointers(const void* A, const void* B, const void* D, int m, in
 }
 
 // Shape -> configuration.  Weights are streamed once, so the only goals are (1) enough
-// workgroups and waves to cover every CU with tens of KB of loads in flight and (2) long
-// contiguous runs per weight row.  Numbers below come from sweeps on one MI355X.
-static Config pick_stream(int m, int n, int k, int cu_count) {
+// loads in flight on every CU to cover HBM latency and (2) long contiguous runs per weight
+// row.  The LDS ring wins wherever it applies (k a multiple of 256); the register-streaming
+// engine covers every other k.  The constants come from sweeps on one MI355X.
+static Config pick_config(int m, int n, int k, int cu_count) {
     Config c;
-    c.engine = ENGINE_DIRECT;
-    c.nt = 1;
     c.mt = m <= 16 ? 1 : 2;
+    c.nt = 1;
+    c.split_k = 1;
+    c.persist = 0;
+    const int tiles16 = (n + 15) / 16;
+    if (k % 256 == 0) {
+        c.engine = ENGINE_LDS;
+        c.ku = 4;
+        const int blocks = k / 256;
+        const int xu0 = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
+        if (tiles16 >= 4 * cu_count) {
+            // many tiles per CU: one persistent workgroup per CU walks them with continuous rings
+            c.rg = 1;
+            c.persist = 1;
+            c.depth = 3;
+            c.waves = 6;
+            while (c.waves > 2 && (size_t)c.waves * (c.depth * (4 + xu0) + 2 * c.mt) * 1024 + 4096 > 159 * 1024)
+                c.waves--;
+            if (c.waves == 5) c.waves = 4;
+        } else {                                // about one tile per CU: few waves, deep rings
+            c.rg = 1;
+            c.waves = blocks >= 48 ? 2 : 1;
+            c.depth = c.waves == 1 ? 8 : 4;
+        }
+        const int xu = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
+        while (c.depth > 2 && ((c.depth - 1) * (c.rg * 4 + xu) > 63 ||
+                               (size_t)c.waves * c.depth * (c.rg * 4 + xu) * 1024 + 4096 > 159 * 1024))
+            c.depth--;
+        if (!c.persist && c.depth > blocks / c.waves && blocks / c.waves >= 2) c.depth = blocks / c.waves;
+        if (c.depth == 5 || c.depth == 7) c.depth--;
+        return c;
+    }
+    c.engine = ENGINE_DIRECT;
     c.ku = (k % 256 == 0) ? 4 : ((k % 128 == 0) ? 2 : 1);
     const int stages = (k + c.ku * 64 - 1) / (c.ku * 64);
-    c.rg = 1;
-    if ((n + 15) / 16 >= 8 * cu_count) c.rg = 2;
+    c.rg = tiles16 >= 8 * cu_count ? 2 : 1;
     const int n_tiles = (n + 16 * c.rg - 1) / (16 * c.rg);
     const int m_tiles = (m + 16 * c.mt - 1) / (16 * c.mt);
     c.waves = stages >= 16 ? 8 : (stages >= 4 ? 4 : (stages >= 2 ? 2 : 1));
-    c.split_k = 1;
-    // few tiles: spread K over more workgroups until every CU has about two of them
+    // few tiles: spread K over more workgroups until half the CUs have one
     while ((long)n_tiles * m_tiles * c.split_k < cu_count / 2 && stages / (c.split_k * 2) >= 2 * c.waves &&
            c.split_k < 16)
         c.split_k *= 2;
@@ -259,6 +298,7 @@ int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* sca
     c.waves = consumers;
     c.split_k = split_k;
     c.nt = 1;
+    c.persist = 0;
     // a 256-byte stage with at least two ring slots is the LDS ring's shape; everything else
     // streams straight into registers
     StreamArgs a{};
@@ -292,7 +332,8 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D, const floa
     c.waves = t->waves;
     c.split_k = t->split_k;
     c.nt = t->non_temporal;
-    if (c.engine == ENGINE_AUTO) c = pick_stream(m, n, k, dev->cu_count);
+    c.persist = t->persistent_wgs_per_cu;
+    if (c.engine == ENGINE_AUTO) c = pick_config(m, n, k, dev->cu_count);
     if (c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
@@ -306,7 +347,7 @@ int sg_skinny_gemm_pick(int m, int n, int k, int out[8]) {
     DeviceInfo* dev;
     int cu = 256;
     if (get_device_info(&dev) == SG_SUCCESS) cu = dev->cu_count;
-    const Config c = pick_stream(m, n, k, cu);
+    const Config c = pick_config(m, n, k, cu);
     const int op_m = c.mt == 2 ? 32 : (m <= 8 ? 8 : 16);
     out[0] = c.split_k; out[1] = 0; out[2] = 0; out[3] = c.waves;
     out[4] = c.rg; out[5] = c.depth; out[6] = op_m; out[7] = c.ku * 64 / (512 / op_m);
@@ -321,7 +362,7 @@ int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D, const float
     if (!scale_tensor) return SG_BAD_ARGUMENT;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const Config c = pick_stream(m, n, k, dev->cu_count);
+    const Config c = pick_config(m, n, k, dev->cu_count);
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
@@ -339,7 +380,7 @@ static int async_gemm_common(const uint8_t* A, const uint8_t* B, void* D, int m,
     if (int rc = check_pointers(A, B, D, m, n, k, k)) return rc;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const Config c = pick_stream(m, n, k, dev->cu_count);
+    const Config c = pick_config(m, n, k, dev->cu_count);
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = nullptr;
     a.m = m; a.n = n; a.k = k; a.b_stride = k;

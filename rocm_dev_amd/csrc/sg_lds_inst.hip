@@ -9,9 +9,9 @@
 
 namespace sg {
 
-template <int XU, int DEPTH, bool NT>
+template <int XU, int DEPTH, bool NT, bool PERSISTENT>
 static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
-    auto kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
+    auto kernel = PERSISTENT ? lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT> : lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
     // dynamic LDS above the default cap must be requested per kernel; remember the largest
     // request made so far on each device
     static size_t attr_bytes[16] = {};
@@ -35,14 +35,17 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
 #define SG_CASE(XU_, DEPTH_)                                                                    \
     if (xu == XU_ && depth == DEPTH_) {                                                         \
         if constexpr ((DEPTH_ - 1) * (SG_RG * 4 + XU_) <= 63 && XU_ <= 4 * SG_MT) {             \
-            return nt ? launch_one<XU_, DEPTH_, true>(a, grid, threads, lds, stream)            \
-                      : launch_one<XU_, DEPTH_, false>(a, grid, threads, lds, stream);          \
+            if (persistent)                                                                     \
+                return nt ? launch_one<XU_, DEPTH_, true, true>(a, grid, threads, lds, stream)  \
+                          : launch_one<XU_, DEPTH_, false, true>(a, grid, threads, lds, stream); \
+            return nt ? launch_one<XU_, DEPTH_, true, false>(a, grid, threads, lds, stream)     \
+                      : launch_one<XU_, DEPTH_, false, false>(a, grid, threads, lds, stream);   \
         } else {                                                                                \
             return SG_INVALID_CONFIG;                                                           \
         }                                                                                       \
     }
 
-int SG_LDS_LAUNCHER(SG_MT, SG_RG)(int xu, int depth, int nt, const StreamArgs& a, unsigned grid, unsigned threads,
+int SG_LDS_LAUNCHER(SG_MT, SG_RG)(int xu, int depth, int nt, int persistent, const StreamArgs& a, unsigned grid, unsigned threads,
                                   size_t lds, hipStream_t stream) {
 #if SG_MT == 1
     SG_CASE(1, 2) SG_CASE(1, 3) SG_CASE(1, 4) SG_CASE(1, 6) SG_CASE(1, 8)

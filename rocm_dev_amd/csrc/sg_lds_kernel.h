@@ -186,4 +186,166 @@ __global__ void __launch_bounds__(1024) lds_gemm_kernel(const StreamArgs a) {
     finish_tile<RG, MT>(a, acc, reinterpret_cast<f32x4*>(ring), &arrival, tile_m, tile_n, split, m0, n0);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Persistent variant for shapes with many more tiles than CUs.  A workgroup walks tiles
+// blockIdx.x, blockIdx.x + gridDim.x, ... and every wave's ring simply continues across the
+// tile boundary: while the waves meet to reduce and store tile j, the DMAs of tile j+1 are
+// already in flight, so HBM never sees the ramp-down / ramp-up of a workgroup hand-over.
+// (The reference's kernel is persistent for the same reason: skinny_gemm_kernel.cu:44-51.)
+// The reduction scratch is double-buffered by tile parity, which leaves one barrier per tile.
+// No cross-workgroup split-K in this variant.
+template <int MT, int RG, int XU, int DEPTH, bool NT>
+__global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamArgs a) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage] then red[2][FRAGS][wave][64]
+
+    constexpr int PER_STAGE = RG * 4 + XU;
+    constexpr int STAGE_BYTES = PER_STAGE * 1024;
+    constexpr int FRAGS = RG * MT;
+    static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
+
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int waves = a.waves;
+    const int r = lane & 15, g = lane >> 4;
+
+    const int total_tiles = a.n_tiles * a.m_tiles;
+    const int my_tiles = ((int)blockIdx.x < total_tiles) ? (total_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    const int blocks = a.k >> 8;
+    const int per_tile = wave < blocks ? (blocks - wave + waves - 1) / waves : 0;
+    const int total = per_tile * my_tiles;
+
+    const int q = lane >> 2, p = lane & 3;
+    const int src_row = q & 3;
+    const int src_col = (q >> 2) * 64;
+    const int rd_off = 1024 * (r >> 2) + 64 * (r & 3) + 16 * ((g - (r >> 2)) & 3);
+    const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
+    const unsigned my_ring_lds = lds_addr(my_ring);
+    f32x4* red = reinterpret_cast<f32x4*>(ring + (size_t)waves * (DEPTH * STAGE_BYTES));
+
+    auto tile_origin = [&](int j, int& m0, int& n0) {  // j-th tile of this workgroup
+        const int t = (int)blockIdx.x + j * (int)gridDim.x;
+        n0 = (t % a.n_tiles) * (16 * RG);
+        m0 = (t / a.n_tiles) * (16 * MT);
+    };
+
+    auto issue = [&](int i) {
+        const int j = i / per_tile;
+        const int kb = wave + (i - j * per_tile) * waves;
+        int m0, n0;
+        tile_origin(j, m0, n0);
+        const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
+        const size_t koff = ((size_t)kb << 8) + src_col;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                int row = n0 + rg * 16 + 4 * u + src_row;
+                row = row < a.n ? row : a.n - 1;
+                const uint8_t* src = a.B + (size_t)row * a.b_stride + koff + ((p + u) & 3) * 16;
+                if (NT) dma_1kb_stream(src, slot + (rg * 4 + u) * 1024);
+                else dma_1kb(src, slot + (rg * 4 + u) * 1024);
+            }
+#pragma unroll
+        for (int u = 0; u < XU; u++) {
+            int row = m0 + 4 * u + src_row;
+            row = row < a.m ? row : a.m - 1;
+            dma_1kb(a.A + (size_t)row * a.k + koff + ((p + (u & 3)) & 3) * 16, slot + (RG * 4 + u) * 1024);
+        }
+    };
+
+    f32x4 acc[RG][MT];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto consume = [&](int i) {
+        const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
+#pragma unroll
+        for (int kc = 0; kc < 4; kc++) {
+            i64x2 x[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+                x[mt] = *reinterpret_cast<const i64x2*>(slot + (RG * 4 + mt * 4) * 1024 + kc * 256);
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                const i64x2 w = *reinterpret_cast<const i64x2*>(slot + rg * 4096 + kc * 256);
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.x, x[mt].x, acc[rg][mt], 0, 0, 0);
+                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.y, x[mt].y, acc[rg][mt], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    const float scale = a.scale ? a.scale[0] : 1.0f;
+    // Reduce the waves' partial tiles of the j-th tile in wave order, scale, round, store.
+    auto tile_done = [&](int j) {
+        int m0, n0;
+        tile_origin(j, m0, n0);
+        if (waves == 1) {
+#pragma unroll
+            for (int f = 0; f < FRAGS; f++)
+                store_fragment(a, acc[f / MT][f % MT], scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g);
+        } else {
+            f32x4* buf = red + (size_t)(j & 1) * (FRAGS * waves * 64);
+#pragma unroll
+            for (int f = 0; f < FRAGS; f++) buf[(f * waves + wave) * 64 + lane] = acc[f / MT][f % MT];
+            __syncthreads();
+            for (int f = wave; f < FRAGS; f += waves) {
+                f32x4 v = buf[(f * waves) * 64 + lane];
+                for (int w = 1; w < waves; w++) v += buf[(f * waves + w) * 64 + lane];
+                store_fragment(a, v, scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g);
+            }
+        }
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    };
+
+    if (per_tile == 0) {  // more waves than K blocks: this wave only takes part in the reductions
+        for (int j = 0; j < my_tiles; j++) tile_done(j);
+        return;
+    }
+
+    // stage i ends a tile when it is this wave's last K block of that tile
+    int left_in_tile = per_tile;  // stages of the current tile not yet consumed
+    int tile_j = 0;
+    auto after_consume = [&]() {
+        if (--left_in_tile == 0) {
+            tile_done(tile_j++);
+            left_in_tile = per_tile;
+        }
+    };
+
+    if (total >= DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) issue(d);
+        int i = 0;
+        for (; i + DEPTH < total; i++) {
+            wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            consume(i);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            issue(i + DEPTH);
+            __builtin_amdgcn_sched_barrier(0);
+            after_consume();
+        }
+        auto consume_and_close = [&](int ii) {
+            consume(ii);
+            after_consume();
+        };
+        drain_ring<0, DEPTH, PER_STAGE>(consume_and_close, i);
+    } else {
+        for (int i = 0; i < total; i++) issue(i);
+        wait_vmcnt<0>();
+        for (int i = 0; i < total; i++) {
+            consume(i);
+            after_consume();
+        }
+    }
+}
+
 }  // namespace sg

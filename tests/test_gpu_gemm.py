@@ -153,6 +153,44 @@ def test_lds_ring_engine(sg, oracle, cfg, shape):
     assert np.array_equal(bits(D2), got)
 
 
+PERSISTENT_CONFIGS = [
+    # waves, row_tiles, depth, persistent workgroups per CU
+    (1, 1, 4, 1),
+    (2, 4, 2, 2),
+    (4, 1, 3, 1),
+    (2, 2, 4, 2),
+    (8, 1, 2, 1),
+    (3, 1, 2, 4),
+]
+
+
+@pytest.mark.parametrize("cfg", PERSISTENT_CONFIGS)
+@pytest.mark.parametrize("shape", [(8, 28672, 1024), (8, 16400, 512), (5, 9000, 768), (16, 6144, 2048), (32, 8192, 1024),
+                                   (3, 128, 512), (40, 12288, 256)])
+def test_lds_ring_persistent(sg, oracle, cfg, shape):
+    """Persistent workgroups walking many tiles with one continuous DMA ring per wave."""
+    waves, row_tiles, depth, per_cu = cfg
+    m, n, k = shape
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=8)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kw = dict(engine=2, waves=waves, row_tiles=row_tiles, depth=depth, persistent_wgs_per_cu=per_cu)
+    rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
+    torch.cuda.synchronize()
+    if rc == 6:
+        pytest.skip("configuration not compiled / does not fit LDS")
+    assert rc == 0, sg.strerror(rc)
+    got = bits(D)
+    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    # the non-persistent kernel sums the same partials in the same order: identical bits
+    D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kw["persistent_wgs_per_cu"] = 0
+    assert sg.skinny_gemm_tuned(A, B, D2, S, **kw) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(D2), got)
+
+
 def test_torch_binding_surface(sg, oracle):
     """HFRK_skinny_gemm as the reference's Python callers use it: B passed as a (k, n) view."""
     m, n, k = 8, 1024, 2048
