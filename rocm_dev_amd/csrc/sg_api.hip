@@ -6,6 +6,7 @@
 
 #include "sg_host.h"
 #include "sg_stream_kernel.h"
+#include "sg_ring_kernel.h"
 #include <string>
 
 namespace sg {
@@ -167,6 +168,52 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     return SG_INVALID_CONFIG;
 }
 
+// Producer/consumer ring: a_producers + b_producers + consumers waves per persistent workgroup.
+struct RingConfig {
+    int mt, b_lanes, qsize, a_producers, b_producers, consumers, nt;
+};
+
+static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
+    if (a.k % 256 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (c.a_producers < 1 || c.b_producers < 1 || c.consumers < 1 || c.qsize < 1) return SG_INVALID_CONFIG;
+    if (c.a_producers + c.b_producers + c.consumers > 16) return SG_TOO_MANY_WARPS;
+    if (c.b_lanes < 1 || c.b_lanes > 6 || (c.mt != 1 && c.mt != 2)) return SG_INVALID_CONFIG;
+    a.waves = c.consumers;
+    a.split_k = 1;
+    a.n_tiles = (a.n + 16 * c.b_lanes - 1) / (16 * c.b_lanes);
+    a.m_tiles = (a.m + 16 * c.mt - 1) / (16 * c.mt);
+    a.ws = nullptr;
+    a.counters = nullptr;
+    const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
+    if (tiles > 0x7fffffffu) return SG_BAD_ARGUMENT;
+    int xu = 8;
+    if (c.mt == 1) {
+        const int need = (a.m + 3) / 4;
+        xu = need <= 1 ? 1 : (need <= 2 ? 2 : 4);
+    }
+    const size_t slot = (size_t)(c.b_lanes * 4 + xu) * 1024;
+    const size_t flags = ((size_t)(2 * c.b_lanes * c.qsize + 2) * sizeof(int) + 1023) & ~(size_t)1023;
+    // ring | double-buffered reduction scratch | flags | 4 KB slack for activation rows that are not loaded
+    const size_t lds = (size_t)c.qsize * slot + 2u * c.b_lanes * c.mt * c.consumers * 1024 + flags + 4096;
+    if (lds > 159 * 1024) return SG_INVALID_CONFIG;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    size_t per_cu = (159 * 1024) / lds;
+    if (per_cu < 1) per_cu = 1;
+    if (per_cu > 4) per_cu = 4;
+    size_t grid = (size_t)dev->cu_count * per_cu;
+    if (grid > tiles) grid = tiles;
+    RingArgs ra;
+    ra.g = a;
+    ra.a_producers = c.a_producers;
+    ra.b_producers = c.b_producers;
+    ra.consumers = c.consumers;
+    ra.qsize = c.qsize;
+    const unsigned threads = (unsigned)(c.a_producers + c.b_producers + c.consumers) * 64;
+    if (c.mt == 1) return SG_RING_LAUNCHER(1)(c.b_lanes, xu, c.nt, ra, (unsigned)grid, threads, lds, stream);
+    return SG_RING_LAUNCHER(2)(c.b_lanes, xu, c.nt, ra, (unsigned)grid, threads, lds, stream);
+}
+
 static int launch_config(const Config& c, const StreamArgs& a, hipStream_t stream) {
     if (c.engine == ENGINE_DIRECT) return launch_stream(c, a, stream);
     if (c.engine == ENGINE_LDS) return launch_lds(c, a, stream);
@@ -287,7 +334,23 @@ int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* sca
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
 
-    if (ring) return SG_INVALID_CONFIG;  // producer/consumer ring variants are dispatched here once compiled in
+    if (ring) {
+        // the ring's stage is one 256-byte K block; both operands need a producer
+        if (warptile_k != 256 || A_producers < 1 || B_producers < 1) return SG_INVALID_CONFIG;
+        RingConfig rc;
+        rc.mt = op_m == 32 ? 2 : 1;
+        rc.b_lanes = b_lanes;
+        rc.qsize = qsize;
+        rc.a_producers = A_producers;
+        rc.b_producers = B_producers;
+        rc.consumers = consumers;
+        rc.nt = 1;
+        StreamArgs ar{};
+        ar.A = A; ar.B = B; ar.D = D; ar.scale = scale_tensor;
+        ar.m = m; ar.n = n; ar.k = k; ar.b_stride = b_stride;
+        ar.out_f32 = 0;
+        return launch_ring(rc, ar, static_cast<hipStream_t>(stream));
+    }
 
     if (warptile_k % 64 != 0) return SG_INVALID_CONFIG;
     Config c;
@@ -375,16 +438,29 @@ int sg_skinny_gemm_fastpath(const uint8_t* A, const uint8_t* B, void* D, const f
     return sg_skinny_gemm_auto(A, B, D, scale_tensor, m, n, k, k, nullptr);
 }
 
+// async_gemm: the producer/consumer ring with a fixed role split (as the reference's
+// async_gemm_* launchers fix theirs in core.cu); shapes the ring cannot take stream directly.
 static int async_gemm_common(const uint8_t* A, const uint8_t* B, void* D, int m, int n, int k, int out_f32) {
     if (k % 64 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (int rc = check_pointers(A, B, D, m, n, k, k)) return rc;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const Config c = pick_config(m, n, k, dev->cu_count);
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = nullptr;
     a.m = m; a.n = n; a.k = k; a.b_stride = k;
     a.out_f32 = out_f32;
+    if (k % 256 == 0) {
+        RingConfig rc;
+        rc.mt = m <= 16 ? 1 : 2;
+        rc.b_lanes = 2;
+        rc.qsize = 6;
+        rc.a_producers = 1;
+        rc.b_producers = 4;
+        rc.consumers = 3;
+        rc.nt = 1;
+        return launch_ring(rc, a, nullptr);
+    }
+    const Config c = pick_config(m, n, k, dev->cu_count);
     return launch_config(c, a, nullptr);
 }
 

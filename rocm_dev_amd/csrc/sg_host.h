@@ -29,6 +29,15 @@ SG_DECL_STREAM(2, 1) SG_DECL_STREAM(2, 2) SG_DECL_STREAM(2, 3) SG_DECL_STREAM(2,
                                 size_t lds, hipStream_t stream);
 SG_DECL_LDS(1, 1) SG_DECL_LDS(1, 2) SG_DECL_LDS(1, 4) SG_DECL_LDS(2, 1) SG_DECL_LDS(2, 2) SG_DECL_LDS(2, 4)
 
+struct RingArgs;
+#define SG_RING_CAT_(a, b) a##b
+#define SG_RING_CAT(a, b) SG_RING_CAT_(a, b)
+#define SG_RING_LAUNCHER(MT) SG_RING_CAT(launch_ring_, MT)
+int SG_RING_LAUNCHER(1)(int bl, int xu, int nt, const RingArgs& ra, unsigned grid, unsigned threads, size_t lds,
+                        hipStream_t stream);
+int SG_RING_LAUNCHER(2)(int bl, int xu, int nt, const RingArgs& ra, unsigned grid, unsigned threads, size_t lds,
+                        hipStream_t stream);
+
 // Prints a HIP failure to stderr when the environment variable SG_VERBOSE is set; returns e.
 hipError_t report_hip(const char* what, hipError_t e);
 

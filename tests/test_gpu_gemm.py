@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import GEMM_TOL, bits, dev, scale_tensor
+from gpu_util import GEMM_TOL, bits, dev, gemm_tol, scale_tensor
 
 pytestmark = pytest.mark.gpu
 
@@ -44,10 +44,11 @@ def test_config1_fastpath(sg, oracle):
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 8, 13, 16, 17, 31, 32])
 def test_m_sweep_small(sg, oracle, m):
-    a8, b8, scale = oracle.make_gemm_operands(m, 512, 1024, seed=m)
+    k = 1024
+    a8, b8, scale = oracle.make_gemm_operands(m, 512, k, seed=m)
     ref = oracle.gemm_omp(a8, b8, scale)
     got = _run_fast(sg, a8, b8, scale)
-    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 30, 64), (5, 18, 272), (16, 1000, 4096 + 16), (32, 34, 48),
@@ -57,7 +58,7 @@ def test_ragged_shapes(sg, oracle, m, n, k):
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=1)
     ref = oracle.gemm_omp(a8, b8, scale)
     got = _run_fast(sg, a8, b8, scale)
-    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
 
 
 def test_b_stride(sg, oracle):
@@ -71,7 +72,7 @@ def test_b_stride(sg, oracle):
     torch.cuda.synchronize()
     got = bits(D)
     assert not np.isnan(oracle.bf16_to_f32(got)).any()
-    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
 
 
 CONFIGS = [
@@ -104,7 +105,7 @@ def test_explicit_configs(sg, oracle, cfg, shape):
     torch.cuda.synchronize()
     assert rc == 0, sg.strerror(rc)
     got = bits(D)
-    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     # a second launch must give the same bits (fixed reduction order, self-resetting counters)
     D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     assert sg.skinny_gemm(A, B, D2, S, split_k, 0, 0, consumers, b_lanes, qsize, op_m, ops) == 0
@@ -145,7 +146,7 @@ def test_lds_ring_engine(sg, oracle, cfg, shape):
         pytest.skip("configuration not compiled / does not fit LDS")
     assert rc == 0, sg.strerror(rc)
     got = bits(D)
-    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     assert sg.skinny_gemm_tuned(A, B, D2, S, engine=2, split_k=split_k, waves=waves, row_tiles=row_tiles, depth=depth,
                                 non_temporal=nt) == 0
@@ -182,13 +183,54 @@ def test_lds_ring_persistent(sg, oracle, cfg, shape):
         pytest.skip("configuration not compiled / does not fit LDS")
     assert rc == 0, sg.strerror(rc)
     got = bits(D)
-    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     # the non-persistent kernel sums the same partials in the same order: identical bits
     D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     kw["persistent_wgs_per_cu"] = 0
     assert sg.skinny_gemm_tuned(A, B, D2, S, **kw) == 0
     torch.cuda.synchronize()
     assert np.array_equal(bits(D2), got)
+
+
+RING_CONFIGS = [
+    # A_producers, B_producers, consumers, b_lanes, qsize
+    (1, 1, 1, 1, 1),
+    (1, 2, 1, 2, 2),
+    (1, 4, 3, 2, 6),
+    (2, 6, 2, 3, 4),
+    (1, 8, 4, 4, 5),
+    (2, 4, 4, 1, 6),
+    (1, 3, 2, 6, 3),
+    (1, 12, 3, 4, 4),
+]
+
+
+@pytest.mark.parametrize("cfg", RING_CONFIGS)
+@pytest.mark.parametrize("shape", [(8, 64, 256), (8, 512, 4096), (16, 8192, 1024), (5, 1000, 2048), (32, 4096, 1024),
+                                   (27, 28672, 512), (40, 2048, 768)])
+def test_producer_consumer_ring(sg, oracle, cfg, shape):
+    """The reference's launcher signature with producers > 0: LDS ring with separate producer and
+    consumer waves, monotone phase flags, persistent tile loop."""
+    ap, bp, cons, bl, qs = cfg
+    m, n, k = shape
+    op_m = 8 if m <= 8 else (16 if m <= 16 else 32)
+    ops = 256 // (512 // op_m)
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=9)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = sg.skinny_gemm(A, B, D, S, 1, ap, bp, cons, bl, qs, op_m, ops)
+    torch.cuda.synchronize()
+    if rc == 6:
+        pytest.skip("ring does not fit LDS")
+    assert rc == 0, sg.strerror(rc)
+    got = bits(D)
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
+    for _ in range(3):   # repeated runs are the reference's race probe (bench.py -t N)
+        D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        assert sg.skinny_gemm(A, B, D2, S, 1, ap, bp, cons, bl, qs, op_m, ops) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(D2), got)
 
 
 def test_torch_binding_surface(sg, oracle):
@@ -203,7 +245,7 @@ def test_torch_binding_surface(sg, oracle):
     rc = op.skinny_gemm_torch_binding(A, W.t(), D, scale_tensor(scale), 1, 0, 0, 4, 2, 2, 4)
     torch.cuda.synchronize()
     assert rc == 0
-    assert oracle.max_rel_err_bf16(bits(D), ref) <= GEMM_TOL
+    assert oracle.max_rel_err_bf16(bits(D), ref) <= gemm_tol(k)
 
 
 def test_invariants_on_device(sg, oracle):
@@ -239,11 +281,12 @@ def test_async_gemm(sg, oracle):
     assert sg.async_gemm(A, B, D32) == 0
     torch.cuda.synchronize()
     got = D32.cpu().numpy()
-    assert np.abs(got - ref32).max() <= 1e-4 * np.abs(ref32).max()
+    # fp32 output: what is left is the MFMA's in-instruction truncation (see gemm_tol) and summation order
+    assert np.abs(got - ref32).max() <= 5e-4 * np.abs(ref32).max()
     Db = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     assert sg.async_gemm(A, B, Db) == 0
     torch.cuda.synchronize()
-    assert oracle.max_rel_err_bf16(bits(Db), oracle.gemm_omp(a8, b8, 1.0)) <= GEMM_TOL
+    assert oracle.max_rel_err_bf16(bits(Db), oracle.gemm_omp(a8, b8, 1.0)) <= gemm_tol(k)
 
 
 @pytest.mark.parametrize("n,k", [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)])
