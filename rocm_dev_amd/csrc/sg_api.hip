@@ -84,7 +84,7 @@ int get_workspace(Workspace** out) {
 }
 
 // ---- kernel dispatch ------------------------------------------------------------------------
-enum Engine { ENGINE_AUTO = 0, ENGINE_DIRECT = 1, ENGINE_LDS = 2, ENGINE_RING = 3 };
+enum Engine { ENGINE_AUTO = 0, ENGINE_DIRECT = 1, ENGINE_LDS = 2, ENGINE_RING = 3, ENGINE_MID = 4 };
 
 struct Config {
     int engine;   // ENGINE_DIRECT: global -> VGPR -> MFMA;  ENGINE_LDS: global -> LDS ring (DMA) -> MFMA
@@ -214,9 +214,60 @@ static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
     return SG_RING_LAUNCHER(2)(c.b_lanes, xu, c.nt, ra, (unsigned)grid, threads, lds, stream);
 }
 
+// Mid-batch engine: c.rg = 16-row weight fragments per wave (2 or 4), c.mt = 16-row activation
+// fragments per wave (2, 4 or 8); a workgroup tile is 32*c.rg weight rows x 32*c.mt activation rows.
+static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) {
+    if (a.k % 128 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if ((c.rg != 2 && c.rg != 4) || (c.mt != 2 && c.mt != 4 && c.mt != 8) || c.depth < 2) return SG_INVALID_CONFIG;
+    const int bn = 32 * c.rg, bm = 32 * c.mt;
+    a.waves = 4;
+    a.split_k = c.split_k;
+    a.n_tiles = (a.n + bn - 1) / bn;
+    a.m_tiles = (a.m + bm - 1) / bm;
+    const int blocks = a.k / 128;
+    if (c.split_k < 1 || c.split_k > blocks) return SG_INVALID_CONFIG;
+    const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
+    if (tiles * c.split_k > 0x7fffffffu) return SG_BAD_ARGUMENT;
+    a.ws = nullptr;
+    a.counters = nullptr;
+    if (c.split_k > 1) {
+        Workspace* w;
+        if (int rc = get_workspace(&w)) return rc;
+        const size_t per_tile = (size_t)4 * c.rg * c.mt * 1024;   // fp32 fragments of one workgroup tile
+        if (tiles > w->n_counters || tiles * c.split_k * per_tile > w->partial_bytes) return SG_WORKSPACE_TOO_SMALL;
+        a.ws = w->partials;
+        a.counters = w->counters;
+    }
+    const size_t lds = (size_t)c.depth * (bn + bm) * 128;
+    if (lds > 159 * 1024) return SG_INVALID_CONFIG;
+    return launch_mid(c.rg, c.mt, c.depth, a, (unsigned)(tiles * c.split_k), lds, stream);
+}
+
+static Config pick_mid(int m, int n, int k, int cu_count) {
+    Config c;
+    c.engine = ENGINE_MID;
+    c.nt = 1;
+    c.persist = 0;
+    c.ku = 2;
+    c.waves = 4;
+    c.mt = m <= 64 ? 2 : (m <= 128 ? 4 : 8);
+    c.rg = (n + 127) / 128 >= cu_count / 2 ? 4 : 2;
+    const int tiles = (n + 32 * c.rg - 1) / (32 * c.rg) * ((m + 32 * c.mt - 1) / (32 * c.mt));
+    const int blocks = k / 128;
+    c.split_k = 1;
+    // few tiles: split K until every CU has a workgroup, keeping at least 16 K blocks per split
+    while (tiles * c.split_k * 2 <= cu_count && blocks / (c.split_k * 2) >= 16 && c.split_k < 8) c.split_k *= 2;
+    c.depth = 6;
+    while (c.depth > 2 && ((size_t)c.depth * (32 * c.rg + 32 * c.mt) * 128 > 159 * 1024 ||
+                           (c.depth - 2) * (c.rg + c.mt) > 63 || c.depth == 5))
+        c.depth--;
+    return c;
+}
+
 static int launch_config(const Config& c, const StreamArgs& a, hipStream_t stream) {
     if (c.engine == ENGINE_DIRECT) return launch_stream(c, a, stream);
     if (c.engine == ENGINE_LDS) return launch_lds(c, a, stream);
+    if (c.engine == ENGINE_MID) return launch_mid_engine(c, a, stream);
     return SG_INVALID_CONFIG;
 }
 
@@ -396,8 +447,9 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D, const floa
     c.split_k = t->split_k;
     c.nt = t->non_temporal;
     c.persist = t->persistent_wgs_per_cu;
-    if (c.engine == ENGINE_AUTO) c = pick_config(m, n, k, dev->cu_count);
-    if (c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
+    if (c.engine == ENGINE_AUTO)
+        c = (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, dev->cu_count) : pick_config(m, n, k, dev->cu_count);
+    if (c.engine != ENGINE_MID && c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
@@ -425,7 +477,7 @@ int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D, const float
     if (!scale_tensor) return SG_BAD_ARGUMENT;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const Config c = pick_config(m, n, k, dev->cu_count);
+    const Config c = (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, dev->cu_count) : pick_config(m, n, k, dev->cu_count);
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;

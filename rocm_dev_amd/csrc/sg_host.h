@@ -38,6 +38,8 @@ int SG_RING_LAUNCHER(1)(int bl, int xu, int nt, const RingArgs& ra, unsigned gri
 int SG_RING_LAUNCHER(2)(int bl, int xu, int nt, const RingArgs& ra, unsigned grid, unsigned threads, size_t lds,
                         hipStream_t stream);
 
+int launch_mid(int rgw, int mh, int depth, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream);
+
 // Prints a HIP failure to stderr when the environment variable SG_VERBOSE is set; returns e.
 hipError_t report_hip(const char* what, hipError_t e);
 

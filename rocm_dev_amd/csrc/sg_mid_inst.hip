@@ -1,0 +1,47 @@
+// Instantiates the mid-batch kernel for every compiled (RGW, MH, DEPTH) and exposes the
+// launcher the dispatcher in sg_api.hip calls.
+#include "sg_mid_kernel.h"
+#include "sg_host.h"
+
+namespace sg {
+
+template <int RGW, int MH, int DEPTH>
+static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
+    auto kernel = mid_gemm_kernel<RGW, MH, DEPTH>;
+    static size_t attr_bytes[16] = {};
+    if (lds > 48 * 1024) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
+        if (attr_bytes[dev] < lds) {
+            if (report_hip("hipFuncSetAttribute",
+                           hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
+                (void)hipGetLastError();
+                return SG_LAUNCH_FAILED;
+            }
+            attr_bytes[dev] = lds;
+        }
+    }
+    kernel<<<dim3(grid), dim3(256), lds, stream>>>(a);
+    return report_hip("mid_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
+}
+
+#define SG_CASE(RGW_, MH_, DEPTH_)                                                     \
+    if (rgw == RGW_ && mh == MH_ && depth == DEPTH_) {                                 \
+        if constexpr ((DEPTH_ - 2) * (RGW_ + MH_) <= 63)                               \
+            return launch_one<RGW_, MH_, DEPTH_>(a, grid, lds, stream);                \
+        else                                                                           \
+            return SG_INVALID_CONFIG;                                                  \
+    }
+
+int launch_mid(int rgw, int mh, int depth, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
+    SG_CASE(2, 2, 2) SG_CASE(2, 2, 3) SG_CASE(2, 2, 4) SG_CASE(2, 2, 6)
+    SG_CASE(2, 4, 2) SG_CASE(2, 4, 3) SG_CASE(2, 4, 4) SG_CASE(2, 4, 6)
+    SG_CASE(2, 8, 2) SG_CASE(2, 8, 3) SG_CASE(2, 8, 4)
+    SG_CASE(4, 2, 2) SG_CASE(4, 2, 3) SG_CASE(4, 2, 4) SG_CASE(4, 2, 6)
+    SG_CASE(4, 4, 2) SG_CASE(4, 4, 3) SG_CASE(4, 4, 4)
+    SG_CASE(4, 8, 2) SG_CASE(4, 8, 3)
+    return SG_INVALID_CONFIG;
+}
+
+}  // namespace sg

@@ -1,0 +1,198 @@
+// Mid-batch FP8 GEMM for gfx950 (32 < M <= 256 per tile):  D[m,n] = scale * sum_k A[m,k] * B[n,k].
+//
+// The skinny kernels cover M <= 32 per pass; the reference handles larger M by looping
+// 32-row tiles, each re-streaming B (skinny_gemm/skinny_gemm_kernel.cu:44-46,54).  Here B is
+// streamed once: a workgroup owns BN = 32*RGW weight rows and ALL activation rows, and both
+// operands of a 128-byte K block are staged in LDS for its four waves.
+//
+// Waves form a 2 x 2 grid over the tile: wave (wn, wm) owns 16*RGW weight rows and 16*MH
+// activation rows, so each weight fragment it reads from LDS feeds MH MFMAs and each
+// activation fragment RGW MFMAs - the register-level reuse that keeps LDS bandwidth (128
+// B/clk/CU) under the MFMA rate.  The MFMA is gfx950's v_mfma_scale_f32_16x16x128_f8f6f4
+// with unit block scales: 128 bytes of K per instruction, i.e. one instruction per stage and
+// fragment pair.  Lane (r = l%16, g = l/16) supplies 32 bytes of row r; which 32 bytes is
+// free as long as both operands agree, so both take 16-byte pieces 2g and 2g+1 of the block.
+//
+// LDS stage layout: row-major, 128 bytes per row, filled by direct-to-LDS loads of 8 rows x
+// 128 contiguous bytes per instruction.  The 16-byte pieces of a row are XOR-swizzled with
+// (row/2) & 7 - a permutation that keeps every aligned 64-byte run intact for the memory
+// system - so the sixteen lanes of a ds_read_b128 pass land in sixteen different bank groups.
+//
+// Pipeline: DEPTH stages in LDS, DEPTH-1 in flight; per K block each wave waits for its own
+// DMAs of that block (s_waitcnt vmcnt), one workgroup barrier publishes the stage and retires
+// the previous one, the freed slot is refilled, the stage is consumed.
+//
+// K is split across workgroups when there are few tiles; partials meet in the fp32 workspace
+// and the last workgroup to arrive sums them in split order (same scheme as the skinny path).
+#pragma once
+
+#include "sg_device.h"
+#include "sg_epilogue.h"
+#include "sg_lds_kernel.h"
+
+namespace sg {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+// RGW: 16-row weight fragments per wave (2 or 4)  -> BN = 32*RGW rows per workgroup
+// MH : 16-row activation fragments per wave (2, 4, 8) -> up to 32*MH activation rows per tile
+template <int RGW, int MH, int DEPTH>
+__global__ void __launch_bounds__(256) mid_gemm_kernel(const StreamArgs a) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [DEPTH][W rows | X rows][128]
+    __shared__ unsigned arrival;
+
+    constexpr int BN = 32 * RGW;
+    constexpr int BM = 32 * MH;
+    constexpr int W_INSTR = BN / 8 / 4;   // DMA instructions per wave per stage for the weights
+    constexpr int X_INSTR = BM / 8 / 4;   // ... and for the activations
+    constexpr int PER_STAGE = W_INSTR + X_INSTR;
+    constexpr int STAGE_BYTES = (BN + BM) * 128;
+    static_assert(DEPTH >= 2 && (DEPTH - 2) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
+
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int wn = wave & 1, wm = wave >> 1;
+
+    int bid = blockIdx.x;
+    const int tile_n = bid % a.n_tiles;
+    bid /= a.n_tiles;
+    const int split = bid % a.split_k;
+    const int tile_m = bid / a.split_k;
+    const int n0 = tile_n * BN;
+    const int m0 = tile_m * BM;
+
+    const int blocks = a.k >> 7;   // 128-byte K blocks
+    const int per_split = blocks / a.split_k;
+    const int b_begin = split * per_split;
+    const int b_end = (split == a.split_k - 1) ? blocks : b_begin + per_split;
+    const int n_blk = b_end - b_begin;
+
+    // ---- DMA sources: instruction i of this wave covers stage rows 8*(4*i + wave) .. +7 ------
+    const int d_row = lane >> 3;                 // row inside the 8-row instruction
+    const int d_pp = lane & 7;                   // physical 16-byte piece inside the 128-byte row
+    const uint8_t* wsrc[W_INSTR];
+    const uint8_t* xsrc[X_INSTR];
+#pragma unroll
+    for (int i = 0; i < W_INSTR; i++) {
+        const int row_l = 8 * (4 * i + wave) + d_row;           // row inside the weight part of the stage
+        int row = n0 + row_l;
+        row = row < a.n ? row : a.n - 1;
+        wsrc[i] = a.B + (size_t)row * a.b_stride + ((d_pp ^ ((row_l >> 1) & 7)) << 4);
+    }
+#pragma unroll
+    for (int i = 0; i < X_INSTR; i++) {
+        const int row_l = 8 * (4 * i + wave) + d_row;
+        int row = m0 + row_l;
+        row = row < a.m ? row : a.m - 1;
+        xsrc[i] = a.A + (size_t)row * a.k + ((d_pp ^ ((row_l >> 1) & 7)) << 4);
+    }
+    const unsigned ring_lds = lds_addr(ring);
+    auto issue = [&](int s) {   // s-th K block of this workgroup -> slot s % DEPTH
+        const size_t koff = (size_t)(b_begin + s) << 7;
+        const unsigned slot = ring_lds + (unsigned)(s % DEPTH) * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < W_INSTR; i++) dma_1kb_stream(wsrc[i] + koff, slot + (4 * i + wave) * 1024);
+#pragma unroll
+        for (int i = 0; i < X_INSTR; i++) dma_1kb(xsrc[i] + koff, slot + BN * 128 + (4 * i + wave) * 1024);
+    };
+
+    // ---- LDS read offsets: lane (r, g) reads pieces 2g and 2g+1 of row r of a 16-row fragment --
+    const int r = lane & 15, g = lane >> 4;
+    const int piece0 = ((2 * g) ^ ((r >> 1) & 7)) << 4;
+    const int rd0 = r * 128 + piece0;
+    const int rd1 = r * 128 + (piece0 ^ 16);
+    const int w_base = (wn * RGW * 16) * 128;                   // this wave's weight rows
+    const int x_base = BN * 128 + (wm * MH * 16) * 128;         // this wave's activation rows
+
+    f32x4 acc[RGW][MH];
+#pragma unroll
+    for (int rg = 0; rg < RGW; rg++)
+#pragma unroll
+        for (int mb = 0; mb < MH; mb++) acc[rg][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto consume = [&](int s) {
+        const uint8_t* slot = ring + (size_t)(s % DEPTH) * STAGE_BYTES;
+        i32x8 x[MH];
+#pragma unroll
+        for (int mb = 0; mb < MH; mb++) {
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(slot + x_base + mb * 2048 + rd0);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(slot + x_base + mb * 2048 + rd1);
+            x[mb] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
+#pragma unroll
+        for (int rg = 0; rg < RGW; rg++) {
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(slot + w_base + rg * 2048 + rd0);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(slot + w_base + rg * 2048 + rd1);
+            const i32x8 w = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+            for (int mb = 0; mb < MH; mb++)
+                // formats 0/0 = OCP E4M3 for both operands; E8M0 scale byte 127 = 2^0 for both
+                acc[rg][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, x[mb], acc[rg][mb], 0, 0, 0, 0x7f7f7f7f,
+                                                                               0, 0x7f7f7f7f);
+        }
+    };
+
+    // ---- pipeline ------------------------------------------------------------------------------
+    const int prologue = n_blk < DEPTH - 1 ? n_blk : DEPTH - 1;
+    for (int s = 0; s < prologue; s++) issue(s);
+    for (int s = 0; s < n_blk; s++) {
+        // stages s .. min(s + DEPTH - 2, n_blk - 1) are in flight; wait for this wave's part of stage s
+        const int younger = (n_blk - 1 - s) < (DEPTH - 2) ? (n_blk - 1 - s) : (DEPTH - 2);
+        if (younger == DEPTH - 2) wait_vmcnt<(DEPTH - 2) * PER_STAGE>();
+        else wait_vmcnt<0>();   // tail of the K range: fewer stages behind this one
+        __syncthreads();        // stage s is complete for every wave; stage s-1 has been consumed by every wave
+        if (s + DEPTH - 1 < n_blk) issue(s + DEPTH - 1);   // refill the slot of stage s-1
+        __builtin_amdgcn_sched_barrier(0);
+        consume(s);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+
+    // ---- epilogue --------------------------------------------------------------------------------
+    const float scale = a.scale ? a.scale[0] : 1.0f;
+    auto store_all = [&](auto&& get) {
+#pragma unroll
+        for (int rg = 0; rg < RGW; rg++)
+#pragma unroll
+            for (int mb = 0; mb < MH; mb++)
+                store_fragment(a, get(rg, mb), scale, m0 + (wm * MH + mb) * 16 + r, n0 + (wn * RGW + rg) * 16 + 4 * g);
+    };
+    if (a.split_k == 1) {
+        store_all([&](int rg, int mb) { return acc[rg][mb]; });
+        return;
+    }
+
+    // split-K: agent-scope partial stores, arrival counter, last workgroup sums in split order
+    constexpr int FRAGS_WG = 4 * RGW * MH;   // fragments of one workgroup tile
+    const int tile_id = tile_m * a.n_tiles + tile_n;
+    float* ws_tile = a.ws + ((size_t)tile_id * a.split_k) * (FRAGS_WG * 256);
+    {
+        float* mine = ws_tile + (size_t)split * (FRAGS_WG * 256) + (size_t)wave * (RGW * MH * 256) + lane;
+#pragma unroll
+        for (int rg = 0; rg < RGW; rg++)
+#pragma unroll
+            for (int mb = 0; mb < MH; mb++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    __hip_atomic_store(mine + (rg * MH + mb) * 256 + e * 64, acc[rg][mb][e], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0)
+        arrival = __hip_atomic_fetch_add(&a.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (arrival != (unsigned)(a.split_k - 1)) return;
+    store_all([&](int rg, int mb) {
+        const float* p = ws_tile + (size_t)wave * (RGW * MH * 256) + (rg * MH + mb) * 256 + lane;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < a.split_k; sp++) {
+            const float* q = p + (size_t)sp * (FRAGS_WG * 256);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] += __hip_atomic_load(q + e * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return v;
+    });
+    if (threadIdx.x == 0) __hip_atomic_store(&a.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace sg

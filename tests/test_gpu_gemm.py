@@ -233,6 +233,72 @@ def test_producer_consumer_ring(sg, oracle, cfg, shape):
         assert np.array_equal(bits(D2), got)
 
 
+MID_CONFIGS = [
+    # row_tiles (RGW), m_blocks (MH), depth, split_k
+    (2, 2, 2, 1),
+    (4, 2, 6, 1),
+    (2, 4, 3, 2),
+    (4, 4, 4, 1),
+    (2, 8, 3, 1),
+    (4, 8, 3, 4),
+    (4, 8, 2, 1),
+]
+
+
+@pytest.mark.parametrize("cfg", MID_CONFIGS)
+@pytest.mark.parametrize("shape", [(64, 512, 1024), (40, 130, 2048), (128, 1024, 2048), (256, 640, 4096), (200, 256, 4096),
+                                   (300, 128, 1536), (33, 64, 128)])
+def test_mid_batch_engine(sg, oracle, cfg, shape):
+    """32 < m: weights streamed once, 2 x 2 waves per tile, 16x16x128 scaled MFMA with unit scales."""
+    rgw, mh, depth, split_k = cfg
+    m, n, k = shape
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=11)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kw = dict(engine=4, split_k=split_k, row_tiles=rgw, m_blocks=mh, depth=depth)
+    rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
+    torch.cuda.synchronize()
+    if rc == 6:
+        pytest.skip("configuration not compiled / does not fit")
+    assert rc == 0, sg.strerror(rc)
+    got = bits(D)
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
+    D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_tuned(A, B, D2, S, **kw) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(D2), got)
+
+
+@pytest.mark.parametrize("m,n,k", [(64, 10240, 8192), (256, 8192, 8192), (128, 57344, 8192), (256, 8192, 28672)])
+def test_mid_batch_config4_shapes(sg, oracle, m, n, k):
+    """BASELINE config 4 shapes at full size through the fastpath.  The oracle checks two
+    512-row slices of the weight matrix (tiles are independent along n); the rest is covered
+    by linearity: doubling the scale doubles every output exactly."""
+    a = oracle.normal_f32((m, k), 0, 1)
+    a8, sa = oracle.quantize_tensor(a)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    w = torch.randn((n, k), generator=g, device="cuda", dtype=torch.float32)
+    sb = w.abs().max() / 448.0
+    B = (w / sb).to(torch.float8_e4m3fn).view(torch.uint8)
+    del w
+    scale = np.float32(sa) * np.float32(sb.item())
+    A, S = dev(a8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_fastpath(A, B, D, S) == 0
+    torch.cuda.synchronize()
+    got = bits(D)
+    for lo in (0, n - 512):
+        b8 = B[lo:lo + 512].cpu().numpy()
+        ref = oracle.gemm_omp(a8, b8, scale)
+        assert oracle.max_rel_err_bf16(got[:, lo:lo + 512], ref) <= GEMM_TOL
+    D2 = torch.empty_like(D)
+    assert sg.skinny_gemm_fastpath(A, B, D2, scale_tensor(2 * scale)) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(D2.float(), 2 * D.float())
+    assert not torch.isnan(D.float()).any()
+
+
 def test_torch_binding_surface(sg, oracle):
     """HFRK_skinny_gemm as the reference's Python callers use it: B passed as a (k, n) view."""
     m, n, k = 8, 1024, 2048
