@@ -128,6 +128,23 @@ int sg_skinny_gemm_pick(int m, int n, int k, int out[8]);
 int sg_async_gemm_f32(const uint8_t* A, const uint8_t* B, float* D, int m, int n, int k);
 int sg_async_gemm_bf16(const uint8_t* A, const uint8_t* B, void* D_bf16, int m, int n, int k);
 
+/* 2:4 structured-sparse FP8 skinny GEMM - no counterpart in the reference (its "sparse" kernels
+ * run dense operands through the sparse instruction, skinny_gemm/consumers/
+ * smfma_16x16x64_consumer.cu:86-92; 2:4-compressed WEIGHTS are new here).
+ *   D[m,n] = bf16( scale[0] * sum_k A[m,k] * Bdense[n,k] ),  Bdense = decompress(B_vals, B_meta)
+ * B_vals [n][k/2]: the two kept E4M3 codes of every group of four consecutive k, in k order.
+ * B_meta [n][k/8]: one nibble per group - low two bits = position (0..3) of the first kept
+ *                  code, high two bits = position of the second (first < second); the group
+ *                  with the lower k sits in the low nibble of each byte.
+ * k must be a multiple of 512, n even; all pointers 16-byte aligned.  The weights are the
+ * sparse operand of gfx950's v_smfmac_f32_16x16x64_fp8_fp8; HBM traffic is 0.625 bytes per
+ * dense weight.  The _tuned form takes row_tiles, waves, depth, split_k and m_blocks from
+ * the record (engine 0 = library's choice). */
+int sg_sparse24_gemm(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D_bf16,
+                     const float* scale_tensor, int m, int n, int k, void* stream);
+int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D_bf16,
+                           const float* scale_tensor, int m, int n, int k, const SgTuning* tuning, void* stream);
+
 /* Replaces  void tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m,
  * int n)  (tiled_sum_reduce/src.cu:52-73):  D[m,n] = sum_b (A[b,m,n] + B[b,m,n]), summed
  * in batch order per element.  Any m, n (the reference needs m % 8 == 0, n % 64 == 0). */

@@ -13,6 +13,8 @@ from .api import (  # noqa: F401
     fp8_encode_rows,
     fp8_reduce_rows,
     skinny_gemm,
+    sparse24_gemm,
+    SgTuning,
     skinny_gemm_fastpath,
     skinny_gemm_pick,
     skinny_gemm_tuned,

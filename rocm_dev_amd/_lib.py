@@ -27,6 +27,8 @@ SIGNATURES = {
     "sg_skinny_gemm_pick": (_i, [_i, _i, _i, C.POINTER(_i * 8)]),
     "sg_async_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i]),
     "sg_async_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i]),
+    "sg_sparse24_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sg_sparse24_gemm_tuned": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "sg_tiled_sum_reduce": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sg_fp8_encode_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "sg_fp8_decode_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),

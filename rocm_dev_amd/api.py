@@ -147,6 +147,21 @@ class HFRK_skinny_gemm:
                                       B_producers, consumers, b_lanes, qsize, op_m, ops, _stream())
 
 
+def sparse24_gemm(A, B_vals, B_meta, D, scale_tensor, tuning=None, check=False):
+    """2:4 sparse weights: B_vals [n, k/2] kept codes, B_meta [n, k/8] position nibbles (include/sgemm.h)."""
+    m, k = A.shape
+    n = B_vals.shape[0]
+    with torch.cuda.device(A.device):
+        if tuning is None:
+            rc = lib.sg_sparse24_gemm(_dev(A, *_FP8), _dev(B_vals, *_FP8), _dev(B_meta, torch.uint8),
+                                      _dev(D, torch.bfloat16), _dev(scale_tensor, torch.float32), m, n, k, _stream())
+        else:
+            rc = lib.sg_sparse24_gemm_tuned(_dev(A, *_FP8), _dev(B_vals, *_FP8), _dev(B_meta, torch.uint8),
+                                            _dev(D, torch.bfloat16), _dev(scale_tensor, torch.float32), m, n, k,
+                                            C.byref(tuning), _stream())
+    return _done(rc, check)
+
+
 def async_gemm(A, B, D, check=False):
     """D = A @ B^T without a scale on the default stream; D is float32 or bfloat16."""
     m, k = A.shape

@@ -7,6 +7,7 @@
 #include "sg_host.h"
 #include "sg_stream_kernel.h"
 #include "sg_ring_kernel.h"
+#include "sg_sparse_kernel.h"
 #include <string>
 
 namespace sg {
@@ -260,6 +261,46 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     c.depth = 6;
     while (c.depth > 2 && ((size_t)c.depth * (32 * c.rg + 32 * c.mt) * 128 > 159 * 1024 ||
                            (c.depth - 2) * (c.rg + c.mt) > 63 || c.depth == 5))
+        c.depth--;
+    return c;
+}
+
+// 2:4 sparse engine: c.rg row tiles per wave, c.waves waves splitting K, c.depth ring slots.
+static int launch_sparse_engine(const Config& c, StreamArgs a, const uint8_t* meta, hipStream_t stream) {
+    if (a.k % 512 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    size_t tiles;
+    if (int rc = prepare(c, a, 512, &tiles)) return rc;
+    int xu2 = 16;
+    if (c.mt == 1) {
+        const int need = (a.m + 3) / 4;
+        xu2 = need <= 1 ? 2 : (need <= 2 ? 4 : 8);
+    }
+    const size_t stage = (size_t)(c.rg * 5 + xu2) * 1024;
+    // + 8 KB: lanes of activation rows that are not loaded read past the last slot
+    const size_t lds = (size_t)c.waves * c.depth * stage + 8192;
+    if (lds > 159 * 1024) return SG_INVALID_CONFIG;
+    SparseArgs sa;
+    sa.g = a;
+    sa.meta = meta;
+    return launch_sparse(c.mt, c.rg, xu2, c.depth, sa, (unsigned)(tiles * c.split_k), (unsigned)c.waves * 64, lds, stream);
+}
+
+static Config pick_sparse(int m, int n, int k, int cu_count) {
+    Config c;
+    c.engine = ENGINE_LDS;
+    c.nt = 1;
+    c.persist = 0;
+    c.ku = 8;
+    c.split_k = 1;
+    c.mt = m <= 16 ? 1 : 2;
+    const int tiles16 = (n + 15) / 16;
+    const int blocks = k / 512;
+    c.rg = tiles16 >= 4 * cu_count ? 2 : 1;
+    c.waves = blocks >= 16 ? 2 : 1;
+    c.depth = 4;
+    const int xu2 = c.mt == 2 ? 16 : ((m + 3) / 4 <= 1 ? 2 : ((m + 3) / 4 <= 2 ? 4 : 8));
+    while (c.depth > 2 && ((c.depth - 1) * (c.rg * 5 + xu2) > 63 ||
+                           (size_t)c.waves * c.depth * (c.rg * 5 + xu2) * 1024 + 8192 > 159 * 1024))
         c.depth--;
     return c;
 }
@@ -523,6 +564,51 @@ int sg_async_gemm_f32(const uint8_t* A, const uint8_t* B, float* D, int m, int n
 
 int sg_async_gemm_bf16(const uint8_t* A, const uint8_t* B, void* D, int m, int n, int k) {
     return async_gemm_common(A, B, D, m, n, k, 0);
+}
+
+int sg_sparse24_gemm(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D, const float* scale_tensor,
+                     int m, int n, int k, void* stream) {
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 512 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (!A || !B_vals || !B_meta || !D || !scale_tensor || m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B_vals) | reinterpret_cast<uintptr_t>(B_meta)) & 15u)
+        return SG_BAD_ALIGNMENT;
+    if (reinterpret_cast<uintptr_t>(D) & 7u) return SG_BAD_ALIGNMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    const Config c = pick_sparse(m, n, k, dev->cu_count);
+    StreamArgs a{};
+    a.A = A; a.B = B_vals; a.D = D; a.scale = scale_tensor;
+    a.m = m; a.n = n; a.k = k; a.b_stride = k / 2;
+    a.out_f32 = 0;
+    return launch_sparse_engine(c, a, B_meta, static_cast<hipStream_t>(stream));
+}
+
+int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D,
+                           const float* scale_tensor, int m, int n, int k, const SgTuning* t, void* stream) {
+    if (!t) return SG_BAD_ARGUMENT;
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 512 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (!A || !B_vals || !B_meta || !D || !scale_tensor || m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B_vals) | reinterpret_cast<uintptr_t>(B_meta)) & 15u)
+        return SG_BAD_ALIGNMENT;
+    if (reinterpret_cast<uintptr_t>(D) & 7u) return SG_BAD_ALIGNMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    Config c = pick_sparse(m, n, k, dev->cu_count);
+    if (t->engine != ENGINE_AUTO) {
+        c.rg = t->row_tiles;
+        c.waves = t->waves;
+        c.depth = t->depth;
+        c.split_k = t->split_k;
+        c.mt = t->m_blocks;
+        if (c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
+    }
+    StreamArgs a{};
+    a.A = A; a.B = B_vals; a.D = D; a.scale = scale_tensor;
+    a.m = m; a.n = n; a.k = k; a.b_stride = k / 2;
+    a.out_f32 = 0;
+    return launch_sparse_engine(c, a, B_meta, static_cast<hipStream_t>(stream));
 }
 
 int sg_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n, void* stream) {

@@ -40,6 +40,10 @@ int SG_RING_LAUNCHER(2)(int bl, int xu, int nt, const RingArgs& ra, unsigned gri
 
 int launch_mid(int rgw, int mh, int depth, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream);
 
+struct SparseArgs;
+int launch_sparse(int mt, int rg, int xu2, int depth, const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds,
+                  hipStream_t stream);
+
 // Prints a HIP failure to stderr when the environment variable SG_VERBOSE is set; returns e.
 hipError_t report_hip(const char* what, hipError_t e);
 

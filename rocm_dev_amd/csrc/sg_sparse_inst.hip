@@ -1,0 +1,47 @@
+// Instantiates the 2:4 sparse kernel for every compiled (MT, RG, XU2, DEPTH) and exposes the
+// launcher the dispatcher in sg_api.hip calls.
+#include "sg_sparse_kernel.h"
+#include "sg_host.h"
+
+namespace sg {
+
+template <int MT, int RG, int XU2, int DEPTH>
+static int launch_one(const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
+    auto kernel = sparse24_gemm_kernel<MT, RG, XU2, DEPTH>;
+    static size_t attr_bytes[16] = {};
+    if (lds > 48 * 1024) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
+        if (attr_bytes[dev] < lds) {
+            if (report_hip("hipFuncSetAttribute",
+                           hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
+                (void)hipGetLastError();
+                return SG_LAUNCH_FAILED;
+            }
+            attr_bytes[dev] = lds;
+        }
+    }
+    kernel<<<dim3(grid), dim3(threads), lds, stream>>>(sa);
+    return report_hip("sparse24_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
+}
+
+#define SG_CASE(MT_, RG_, XU2_, DEPTH_)                                                     \
+    if (mt == MT_ && rg == RG_ && xu2 == XU2_ && depth == DEPTH_) {                          \
+        if constexpr ((DEPTH_ - 1) * (RG_ * 5 + XU2_) <= 63)                                \
+            return launch_one<MT_, RG_, XU2_, DEPTH_>(sa, grid, threads, lds, stream);      \
+        else                                                                                \
+            return SG_INVALID_CONFIG;                                                       \
+    }
+#define SG_DEPTHS(MT_, RG_, XU2_) SG_CASE(MT_, RG_, XU2_, 2) SG_CASE(MT_, RG_, XU2_, 3) SG_CASE(MT_, RG_, XU2_, 4) SG_CASE(MT_, RG_, XU2_, 6)
+
+int launch_sparse(int mt, int rg, int xu2, int depth, const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds,
+                  hipStream_t stream) {
+    SG_DEPTHS(1, 1, 2) SG_DEPTHS(1, 1, 4) SG_DEPTHS(1, 1, 8)
+    SG_DEPTHS(1, 2, 2) SG_DEPTHS(1, 2, 4) SG_DEPTHS(1, 2, 8)
+    SG_DEPTHS(1, 4, 2) SG_DEPTHS(1, 4, 4) SG_DEPTHS(1, 4, 8)
+    SG_DEPTHS(2, 1, 16) SG_DEPTHS(2, 2, 16) SG_DEPTHS(2, 4, 16)
+    return SG_INVALID_CONFIG;
+}
+
+}  // namespace sg

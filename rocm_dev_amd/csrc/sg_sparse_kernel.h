@@ -1,0 +1,173 @@
+// 2:4 structured-sparse FP8 skinny GEMM for gfx950:
+//     D[m,n] = scale * sum_k A[m,k] * Bdense[n,k],   Bdense = decompress(vals, meta)
+// with the weights stored compressed: vals[n][k/2] (the two kept E4M3 codes of every group of
+// four consecutive k) and meta[n][k/8] (one nibble per group: low two bits = position of the
+// first kept value, high two bits = position of the second; group 2u in the low nibble of
+// byte u).  No counterpart in the reference: its "sparse" kernels feed a DENSE activation tile
+// through the sparse instruction (skinny_gemm/consumers/smfma_16x16x64_consumer.cu:86-92);
+// here the compressed WEIGHTS are the sparse operand, which is what the instruction is for.
+//
+// v_smfmac_f32_16x16x64_fp8_fp8: first operand 16 sparse rows (weight rows n) x 64 dense k,
+// of which lane (r = l%16, g = l/16) supplies the 8 stored bytes of its 16-k window plus 16
+// index bits; second operand 16 columns (activation rows m) x 64 k, lane (c, g) supplying the
+// 16 dense bytes of the same window.  The window a lane works on is free as long as both
+// operands agree, so per 512-k stage lane g owns k range [128 g, 128 g + 128): 64 contiguous
+// stored bytes, 16 contiguous metadata bytes and 128 contiguous activation bytes, consumed in
+// eight steps of 16 k.  Per step the index bits are two metadata bytes, already in the order
+// the instruction wants (group j of the window in bits 4j..4j+3).
+//
+// Streaming: same direct-to-LDS ring as the dense kernel (sg_lds_kernel.h) - 4 rows x 256
+// contiguous bytes per DMA instruction for values and activations, 16 rows x 64 bytes for the
+// metadata - with the 16-byte pieces of each row XOR-swizzled by the row number so that all
+// LDS reads are conflict-free.  HBM traffic per weight row is 0.625 bytes per dense k.
+#pragma once
+
+#include "sg_device.h"
+#include "sg_epilogue.h"
+#include "sg_lds_kernel.h"
+
+namespace sg {
+
+struct SparseArgs {
+    StreamArgs g;          // g.B = vals (row stride k/2); shapes as for the dense kernels
+    const uint8_t* meta;   // [n][k/8]
+};
+
+// XU2 = activation DMA instructions per stage: 2 halves x ceil(rows/4)
+template <int MT, int RG, int XU2, int DEPTH>
+__global__ void __launch_bounds__(1024) sparse24_gemm_kernel(const SparseArgs sa) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
+    __shared__ unsigned arrival;
+    const StreamArgs& a = sa.g;
+
+    constexpr int PER_STAGE = RG * 5 + XU2;   // DMA instructions per stage
+    constexpr int STAGE_BYTES = PER_STAGE * 1024;
+    constexpr int X_OFF = RG * 5 * 1024;      // stage: [rg: 4 KB values | 1 KB metadata] ... | activations
+    static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
+    static_assert(XU2 <= 8 * MT, "more activation rows than the tile has");
+
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int waves = a.waves;
+
+    int bid = blockIdx.x;
+    const int tile_n = bid % a.n_tiles;
+    bid /= a.n_tiles;
+    const int split = bid % a.split_k;
+    const int tile_m = bid / a.split_k;
+    const int n0 = tile_n * (16 * RG);
+    const int m0 = tile_m * (16 * MT);
+
+    const int blocks = a.k >> 9;   // 512-k stages
+    const int per_split = blocks / a.split_k;
+    const int b_begin = split * per_split;
+    const int b_end = (split == a.split_k - 1) ? blocks : b_begin + per_split;
+    const int n_blk = b_end - b_begin;
+    const int mine = wave < n_blk ? (n_blk - wave + waves - 1) / waves : 0;
+
+    // ---- DMA sources ------------------------------------------------------------------------
+    const int v_row = lane >> 4, v_pp = lane & 15;     // values / activations: 4 rows x 16 pieces
+    const int t_row = lane >> 2, t_pp = lane & 3;      // metadata: 16 rows x 4 pieces
+    const size_t v_stride = (size_t)(a.k >> 1), t_stride = (size_t)(a.k >> 3);
+    const uint8_t* vsrc[RG][4];
+    const uint8_t* tsrc[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int row16 = 4 * u + v_row;
+            int row = n0 + rg * 16 + row16;
+            row = row < a.n ? row : a.n - 1;
+            vsrc[rg][u] = a.B + (size_t)row * v_stride + ((v_pp ^ row16) << 4);
+        }
+        int row = n0 + rg * 16 + t_row;
+        row = row < a.n ? row : a.n - 1;
+        tsrc[rg] = sa.meta + (size_t)row * t_stride + ((t_pp ^ (t_row >> 2)) << 4);
+    }
+    const uint8_t* xsrc[XU2];
+#pragma unroll
+    for (int i = 0; i < XU2; i++) {
+        const int row_l = 4 * (i >> 1) + v_row;          // row inside the activation tile
+        int row = m0 + row_l;
+        row = row < a.m ? row : a.m - 1;
+        xsrc[i] = a.A + (size_t)row * a.k + (i & 1) * 256 + ((v_pp ^ (row_l & 15)) << 4);
+    }
+
+    const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
+    const unsigned my_ring_lds = lds_addr(my_ring);
+    auto issue = [&](int i) {
+        const size_t kb = (size_t)(b_begin + wave + i * waves);
+        const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) dma_1kb_stream(vsrc[rg][u] + (kb << 8), slot + (rg * 5 + u) * 1024);
+            dma_1kb_stream(tsrc[rg] + (kb << 6), slot + (rg * 5 + 4) * 1024);
+        }
+#pragma unroll
+        for (int i2 = 0; i2 < XU2; i2++) dma_1kb(xsrc[i2] + (kb << 9), slot + X_OFF + i2 * 1024);
+    };
+
+    // ---- LDS read offsets ---------------------------------------------------------------------
+    const int r = lane & 15, g = lane >> 4;
+    const int v_rd = (r >> 2) * 1024 + (r & 3) * 256;                               // + ((4g + i) ^ r) * 16
+    const int t_rd = 4096 + r * 64 + ((g ^ (r >> 2)) << 4);
+    const int x_rd = ((r >> 2) * 2 + (g >> 1)) * 1024 + (r & 3) * 256;              // + ((8(g&1) + t) ^ r) * 16
+
+    f32x4 acc[RG][MT];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto consume = [&](int i) {
+        const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES;
+        i32x4 x[MT][8];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+                x[mt][t] = *reinterpret_cast<const i32x4*>(slot + X_OFF + mt * 8192 + x_rd + (((8 * (g & 1) + t) ^ r) << 4));
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const uint8_t* w = slot + rg * 5120;
+            const i32x4 idx = *reinterpret_cast<const i32x4*>(w + t_rd);
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const i32x4 v = *reinterpret_cast<const i32x4*>(w + v_rd + (((4 * g + p) ^ r) << 4));
+                const i32x2 v_lo = {v.x, v.y}, v_hi = {v.z, v.w};
+                const int id_lo = idx[p] & 0xffff, id_hi = (unsigned)idx[p] >> 16;
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    acc[rg][mt] = __builtin_amdgcn_smfmac_f32_16x16x64_fp8_fp8(v_lo, x[mt][2 * p], acc[rg][mt], id_lo, 0, 0);
+                    acc[rg][mt] = __builtin_amdgcn_smfmac_f32_16x16x64_fp8_fp8(v_hi, x[mt][2 * p + 1], acc[rg][mt], id_hi, 0, 0);
+                }
+            }
+        }
+    };
+
+    if (mine >= DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; d++) issue(d);
+        int i = 0;
+        for (; i + DEPTH < mine; i++) {
+            wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            consume(i);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            issue(i + DEPTH);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        drain_ring<0, DEPTH, PER_STAGE>(consume, i);
+    } else {
+        for (int i = 0; i < mine; i++) issue(i);
+        wait_vmcnt<0>();
+        for (int i = 0; i < mine; i++) consume(i);
+    }
+
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    finish_tile<RG, MT>(a, acc, reinterpret_cast<f32x4*>(ring), &arrival, tile_m, tile_n, split, m0, n0);
+}
+
+}  // namespace sg
