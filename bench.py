@@ -186,6 +186,85 @@ def main():
                               "us": round(mean_us, 3), "TBps": round(nb / mean_us / 1e6, 3),
                               "frac_peak": round(nb / mean_us / 1e6 / 8.0, 4)})
 
+    # ---- the other configurations of the path, one timing each (not part of `value`) ---------
+    def graph_time_us(fn, reps):
+        with torch.cuda.stream(side):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                st = torch.cuda.current_stream().cuda_stream
+                for i in range(reps):
+                    fn(i, st)
+            g.replay()
+            torch.cuda.synchronize()
+            best = 1e30
+            for _ in range(3):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                g.replay()
+                b.record()
+                torch.cuda.synchronize()
+                best = min(best, a.elapsed_time(b) * 1e3 / reps)
+        return best
+
+    others = None
+    if not args.no_sweep:
+        others = {}
+        # per-row FP8 codec, 8192 x 8192 (encode bf16 -> e4m3 + row scales; decode + reduce of 8 buffers)
+        rows = cols = 8192
+        xs = [torch.randn((rows, cols), device="cuda").bfloat16() for _ in range(4)]      # 4 x 128 MiB, rotated
+        q8 = torch.empty((8, rows, cols), device="cuda", dtype=torch.uint8)
+        s8 = torch.empty((8, rows), device="cuda", dtype=torch.float32)
+        y = torch.empty((rows, cols), device="cuda", dtype=torch.bfloat16)
+        for i in range(8):
+            lib.sg_fp8_encode_rows(xs[i % 4].data_ptr(), q8[i].data_ptr(), s8[i].data_ptr(), rows, cols, None)
+        torch.cuda.synchronize()
+        enc_us = graph_time_us(lambda i, st: lib.sg_fp8_encode_rows(xs[i % 4].data_ptr(), q8[i % 8].data_ptr(),
+                                                                    s8[i % 8].data_ptr(), rows, cols, st), 16)
+        dec_us = graph_time_us(lambda i, st: lib.sg_fp8_decode_rows(q8[i % 8].data_ptr(), s8[i % 8].data_ptr(),
+                                                                    y.data_ptr(), rows, cols, st), 16)
+        red_us = graph_time_us(lambda i, st: lib.sg_fp8_reduce_rows(q8.data_ptr(), s8.data_ptr(), y.data_ptr(), 8,
+                                                                    rows * cols, rows, cols, st), 8)
+        enc_b, dec_b, red_b = 3 * rows * cols + 4 * rows, 3 * rows * cols + 4 * rows, 8 * (rows * cols + 4 * rows) + 2 * rows * cols
+        others["fp8_codec_8192x8192"] = {
+            "encode_us": round(enc_us, 2), "encode_TBps": round(enc_b / enc_us / 1e6, 3),
+            "decode_us": round(dec_us, 2), "decode_TBps": round(dec_b / dec_us / 1e6, 3),
+            "reduce8_us": round(red_us, 2), "reduce8_TBps": round(red_b / red_us / 1e6, 3),
+            "note": "reduce reads 512 MiB per launch; the 8 encoded buffers are re-read every launch (beyond the 256 MB cache)"}
+        del xs, q8, s8, y
+        # mid-batch GEMMs (Llama-3-70B-sized layers)
+        mid = []
+        for (n, k) in ((10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)):
+            copies = max(2, int(COLD_BYTES // (n * k)) + 1)
+            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(copies)]
+            for m in (64, 128, 256):
+                a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+                d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+                one = torch.ones(1, device="cuda")
+                us = graph_time_us(lambda i, st: lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(),
+                                                                         one.data_ptr(), m, n, k, k, st), 2 * copies)
+                mid.append({"m": m, "n": n, "k": k, "us": round(us, 2), "TBps": round(gemm_bytes(m, n, k) / us / 1e6, 3),
+                            "TFLOPs": round(2.0 * m * n * k / us / 1e6, 1), "frac_fp8_peak": round(2.0 * m * n * k / us / 1e6 / 5000.0, 4)})
+            del wb
+        others["mid_batch"] = mid
+        # 2:4 sparse GEMMs
+        sp = []
+        nib = torch.tensor([0x4, 0x8, 0xC, 0x9, 0xD, 0xE], dtype=torch.uint8, device="cuda")
+        for (n, k) in ((4096, 14336), (14336, 4096)):
+            copies = max(2, int(COLD_BYTES // (n * k * 0.625)) + 1)
+            vb = [torch.randint(0, 0x7E, (n, k // 2), device="cuda", dtype=torch.uint8) for _ in range(copies)]
+            mb = [(nib[torch.randint(0, 6, (n, k // 8), device="cuda")] | (nib[torch.randint(0, 6, (n, k // 8), device="cuda")] << 4))
+                  for _ in range(copies)]
+            for m in (1, 8, 16, 32):
+                a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+                d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+                one = torch.ones(1, device="cuda")
+                us = graph_time_us(lambda i, st: lib.sg_sparse24_gemm(a8.data_ptr(), vb[i % copies].data_ptr(), mb[i % copies].data_ptr(),
+                                                                      d.data_ptr(), one.data_ptr(), m, n, k, st), 2 * copies)
+                nb = m * k + 0.625 * n * k + 2 * m * n
+                sp.append({"m": m, "n": n, "k": k, "us": round(us, 2), "TBps": round(nb / us / 1e6, 3)})
+            del vb, mb
+        others["sparse24"] = sp
+
     # ---- CPU baseline: the oracle's all-core loop on the same step (rank 0, N = 1 only) ------
     cpu = None
     if not args.no_cpu:
@@ -220,7 +299,7 @@ def main():
                    "(rotating buffers > 2x MALL)" % args.m, "step_bytes": step_bytes,
                    "us_per_gemm_in_step": round(ms_per_step * 1e3 / 4, 3), "frac_hbm_peak": round(value_tbs / 8.0, 4),
                    "host_wall_ms": round((t_host1 - t_host0) * 1e3, 3)},
-        "roofline": roofline, "cpu_baseline": cpu, "per_shape": per_shape, "sweep": sweep,
+        "roofline": roofline, "cpu_baseline": cpu, "per_shape": per_shape, "sweep": sweep, "other_configs": others,
     }
     print(json.dumps(out))
 
