@@ -111,6 +111,9 @@ typedef struct SgTuning {
     int k_chunks;      /* direct engine: 64-byte K chunks per stage (1, 2, 4, 8); LDS ring: fixed 256-byte stage */
     int non_temporal;  /* LDS ring: stream weights with the non-temporal hint */
     int persistent_wgs_per_cu; /* LDS ring: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU */
+    int wave_tiles;    /* LDS ring: 1 = every wavefront owns whole tiles over the full K range and the activations
+                          stay resident in LDS; 2 = persistent K-split workgroups with resident activations
+                          (both need persistent_wgs_per_cu >= 1, split_k = 1, m <= 16*m_blocks) */
 } SgTuning;
 
 int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,

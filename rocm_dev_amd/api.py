@@ -93,20 +93,20 @@ class SgTuning(C.Structure):
     """Mirror of the C struct SgTuning (include/sgemm.h)."""
     _fields_ = [(name, C.c_int) for name in
                 ("engine", "split_k", "waves", "row_tiles", "m_blocks", "depth", "k_chunks", "non_temporal",
-                 "persistent_wgs_per_cu")]
+                 "persistent_wgs_per_cu", "wave_tiles")]
 
 
 ENGINE_AUTO, ENGINE_DIRECT, ENGINE_LDS = 0, 1, 2
 
 
 def skinny_gemm_tuned(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k=1, waves=4, row_tiles=1, m_blocks=None,
-                      depth=2, k_chunks=4, non_temporal=1, persistent_wgs_per_cu=0, check=False):
+                      depth=2, k_chunks=4, non_temporal=1, persistent_wgs_per_cu=0, wave_tiles=0, check=False):
     """The library-native tuning entry (no reference counterpart): pick the engine and its shape."""
     m, k = A.shape
     n = B.shape[0]
     if m_blocks is None:
         m_blocks = 1 if m <= 16 else 2
-    t = SgTuning(engine, split_k, waves, row_tiles, m_blocks, depth, k_chunks, non_temporal, persistent_wgs_per_cu)
+    t = SgTuning(engine, split_k, waves, row_tiles, m_blocks, depth, k_chunks, non_temporal, persistent_wgs_per_cu, wave_tiles)
     with torch.cuda.device(A.device):
         rc = lib.sg_skinny_gemm_tuned(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
                                       _dev(scale_tensor, torch.float32), m, n, k, B.stride(0), C.byref(t), _stream())

@@ -97,6 +97,8 @@ struct Config {
     int split_k;  // workgroups per tile, splitting K among themselves
     int nt;       // weights loaded with the non-temporal hint
     int persist;  // LDS engine: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU walking the tiles
+    int wavetile; // LDS engine: 1 = every wave owns whole tiles, activations resident in LDS (persist = workgroups per CU);
+                  //             2 = persistent K-split workgroups with the activations resident in LDS
 };
 
 static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out) {
@@ -151,8 +153,26 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     // + 4 KB: lanes of activation rows that are not loaded read past the last slot
     size_t lds = (size_t)c.waves * c.depth * stage + 4096;
     unsigned grid = (unsigned)(tiles * c.split_k);
-    if (c.persist > 0) {
+    int mode = 0;
+    if (c.wavetile == 1) {
+        // whole activation matrix resident: one tile row of activations only, no K split
+        if (c.split_k != 1 || a.m_tiles != 1 || c.persist < 1) return SG_INVALID_CONFIG;
+        mode = 2;
+        lds = (size_t)(a.k / 256) * xu * 1024 + (size_t)c.waves * c.depth * c.rg * 4096 + 4096;
+        DeviceInfo* dev;
+        if (int rc = get_device_info(&dev)) return rc;
+        size_t want = (tiles + c.waves - 1) / c.waves;
+        const size_t cap = (size_t)dev->cu_count * c.persist;
+        if (want > cap) want = cap;
+        grid = (unsigned)want;
+    } else if (c.persist > 0) {
         if (c.split_k != 1) return SG_INVALID_CONFIG;
+        mode = 1;
+        if (c.wavetile == 2) {   // activations resident: stages hold weights only
+            if (a.m_tiles != 1) return SG_INVALID_CONFIG;
+            mode = 3;
+            lds = (size_t)(a.k / 256) * xu * 1024 + (size_t)c.waves * c.depth * c.rg * 4096 + 4096;
+        }
         lds += 2u * c.waves * c.rg * c.mt * 1024;   // double-buffered reduction scratch
         DeviceInfo* dev;
         if (int rc = get_device_info(&dev)) return rc;
@@ -163,7 +183,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     const unsigned threads = (unsigned)c.waves * 64;
 #define SG_GO(MT, RG)                                                                                          \
     if (c.mt == MT && c.rg == RG)                                                                              \
-        return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, c.persist > 0, a, grid, threads, lds, stream);
+        return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, mode, a, grid, threads, lds, stream);
     SG_GO(1, 1) SG_GO(1, 2) SG_GO(1, 4) SG_GO(2, 1) SG_GO(2, 2) SG_GO(2, 4)
 #undef SG_GO
     return SG_INVALID_CONFIG;
@@ -249,6 +269,7 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     c.engine = ENGINE_MID;
     c.nt = 1;
     c.persist = 0;
+    c.wavetile = 0;
     c.ku = 2;
     c.waves = 4;
     c.mt = m <= 64 ? 2 : (m <= 128 ? 4 : 8);
@@ -290,6 +311,7 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
     c.engine = ENGINE_LDS;
     c.nt = 1;
     c.persist = 0;
+    c.wavetile = 0;
     c.ku = 8;
     c.split_k = 1;
     c.mt = m <= 16 ? 1 : 2;
@@ -330,16 +352,26 @@ static Config pick_config(int m, int n, int k, int cu_count) {
     c.nt = 1;
     c.split_k = 1;
     c.persist = 0;
+    c.wavetile = 0;
     const int tiles16 = (n + 15) / 16;
     if (k % 256 == 0) {
         c.engine = ENGINE_LDS;
         c.ku = 4;
         const int blocks = k / 256;
         const int xu0 = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
-        if (tiles16 >= 4 * cu_count) {
-            // many tiles per CU: one persistent workgroup per CU walks them with continuous rings
+        if (tiles16 >= 2 * cu_count) {
+            // several tiles per CU: one persistent workgroup per CU walks them with continuous rings;
+            // when one activation tile covers all of m, it stays resident in LDS and the stages
+            // carry weights only
             c.rg = 1;
             c.persist = 1;
+            const size_t x_res = (size_t)blocks * xu0 * 1024;
+            c.waves = m <= 8 ? 8 : 6;
+            c.depth = 2;
+            if (m <= 16 * c.mt && x_res + (size_t)c.waves * (c.depth * 4 + 2 * c.mt) * 1024 + 4096 <= 159 * 1024) {
+                c.wavetile = 2;
+                return c;
+            }
             c.depth = 3;
             c.waves = 6;
             while (c.waves > 2 && (size_t)c.waves * (c.depth * (4 + xu0) + 2 * c.mt) * 1024 + 4096 > 159 * 1024)
@@ -455,6 +487,7 @@ int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* sca
     c.split_k = split_k;
     c.nt = 1;
     c.persist = 0;
+    c.wavetile = 0;
     // a 256-byte stage with at least two ring slots is the LDS ring's shape; everything else
     // streams straight into registers
     StreamArgs a{};
@@ -489,6 +522,7 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D, const floa
     c.split_k = t->split_k;
     c.nt = t->non_temporal;
     c.persist = t->persistent_wgs_per_cu;
+    c.wavetile = t->wave_tiles;
     if (c.engine == ENGINE_AUTO)
         c = (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, dev->cu_count) : pick_config(m, n, k, dev->cu_count);
     if (c.engine != ENGINE_MID && c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;

@@ -25,7 +25,7 @@ SG_DECL_STREAM(2, 1) SG_DECL_STREAM(2, 2) SG_DECL_STREAM(2, 3) SG_DECL_STREAM(2,
 #define SG_CAT_LDS(a, b, c) SG_CAT_LDS_(a, b, c)
 #define SG_LDS_LAUNCHER(MT, RG) SG_CAT_LDS(launch_lds_, MT, RG)
 #define SG_DECL_LDS(MT, RG)                                                                              \
-    int SG_LDS_LAUNCHER(MT, RG)(int xu, int depth, int nt, int persistent, const StreamArgs& a, unsigned grid, unsigned threads, \
+    int SG_LDS_LAUNCHER(MT, RG)(int xu, int depth, int nt, int mode, const StreamArgs& a, unsigned grid, unsigned threads, \
                                 size_t lds, hipStream_t stream);
 SG_DECL_LDS(1, 1) SG_DECL_LDS(1, 2) SG_DECL_LDS(1, 4) SG_DECL_LDS(2, 1) SG_DECL_LDS(2, 2) SG_DECL_LDS(2, 4)
 

@@ -9,9 +9,13 @@
 
 namespace sg {
 
-template <int XU, int DEPTH, bool NT, bool PERSISTENT>
+template <int XU, int DEPTH, bool NT, int MODE>
 static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
-    auto kernel = PERSISTENT ? lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT> : lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
+    void (*kernel)(const StreamArgs) = nullptr;
+    if constexpr (MODE == 2) kernel = lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
+    else if constexpr (MODE == 3) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
+    else if constexpr (MODE == 1) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false>;
+    else kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
     // dynamic LDS above the default cap must be requested per kernel; remember the largest
     // request made so far on each device
     static size_t attr_bytes[16] = {};
@@ -34,18 +38,33 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
 
 #define SG_CASE(XU_, DEPTH_)                                                                    \
     if (xu == XU_ && depth == DEPTH_) {                                                         \
-        if constexpr ((DEPTH_ - 1) * (SG_RG * 4 + XU_) <= 63 && XU_ <= 4 * SG_MT) {             \
-            if (persistent)                                                                     \
-                return nt ? launch_one<XU_, DEPTH_, true, true>(a, grid, threads, lds, stream)  \
-                          : launch_one<XU_, DEPTH_, false, true>(a, grid, threads, lds, stream); \
-            return nt ? launch_one<XU_, DEPTH_, true, false>(a, grid, threads, lds, stream)     \
-                      : launch_one<XU_, DEPTH_, false, false>(a, grid, threads, lds, stream);   \
+        if constexpr (XU_ <= 4 * SG_MT && (SG_MT == 1 || XU_ > 4)) {                            \
+            if (mode == 2 || mode == 3) {                                                       \
+                if constexpr ((DEPTH_ - 1) * (SG_RG * 4) <= 63) {                               \
+                    if (mode == 3)                                                              \
+                        return nt ? launch_one<XU_, DEPTH_, true, 3>(a, grid, threads, lds, stream) \
+                                  : launch_one<XU_, DEPTH_, false, 3>(a, grid, threads, lds, stream); \
+                    return nt ? launch_one<XU_, DEPTH_, true, 2>(a, grid, threads, lds, stream) \
+                              : launch_one<XU_, DEPTH_, false, 2>(a, grid, threads, lds, stream); \
+                } else {                                                                        \
+                    return SG_INVALID_CONFIG;                                                   \
+                }                                                                               \
+            }                                                                                   \
+            if constexpr ((DEPTH_ - 1) * (SG_RG * 4 + XU_) <= 63) {                             \
+                if (mode == 1)                                                                  \
+                    return nt ? launch_one<XU_, DEPTH_, true, 1>(a, grid, threads, lds, stream) \
+                              : launch_one<XU_, DEPTH_, false, 1>(a, grid, threads, lds, stream); \
+                return nt ? launch_one<XU_, DEPTH_, true, 0>(a, grid, threads, lds, stream)     \
+                          : launch_one<XU_, DEPTH_, false, 0>(a, grid, threads, lds, stream);   \
+            } else {                                                                            \
+                return SG_INVALID_CONFIG;                                                       \
+            }                                                                                   \
         } else {                                                                                \
             return SG_INVALID_CONFIG;                                                           \
         }                                                                                       \
     }
 
-int SG_LDS_LAUNCHER(SG_MT, SG_RG)(int xu, int depth, int nt, int persistent, const StreamArgs& a, unsigned grid, unsigned threads,
+int SG_LDS_LAUNCHER(SG_MT, SG_RG)(int xu, int depth, int nt, int mode, const StreamArgs& a, unsigned grid, unsigned threads,
                                   size_t lds, hipStream_t stream) {
 #if SG_MT == 1
     SG_CASE(1, 2) SG_CASE(1, 3) SG_CASE(1, 4) SG_CASE(1, 6) SG_CASE(1, 8)

@@ -53,6 +53,18 @@ __device__ __forceinline__ void wait_vmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+// waits until at most n (a run-time value, clamped to 63) vector-memory operations are outstanding
+__device__ __forceinline__ void wait_vmcnt_upto(int n) {
+    if (n >= 48) wait_vmcnt<48>();
+    else if (n >= 32) wait_vmcnt<32>();
+    else if (n >= 24) wait_vmcnt<24>();
+    else if (n >= 16) wait_vmcnt<16>();
+    else if (n >= 12) wait_vmcnt<12>();
+    else if (n >= 8) wait_vmcnt<8>();
+    else if (n >= 4) wait_vmcnt<4>();
+    else wait_vmcnt<0>();
+}
+
 // Drains the last DEPTH stages: stage D of them still has DEPTH-1-D younger stages in flight.
 template <int D, int DEPTH, int PER_STAGE, class Consume>
 __device__ __forceinline__ void drain_ring(Consume& consume, int i) {
@@ -196,11 +208,12 @@ __global__ void __launch_bounds__(1024) lds_gemm_kernel(const StreamArgs a) {
 // (The reference's kernel is persistent for the same reason: skinny_gemm_kernel.cu:44-51.)
 // The reduction scratch is double-buffered by tile parity, which leaves one barrier per tile.
 // No cross-workgroup split-K in this variant.
-template <int MT, int RG, int XU, int DEPTH, bool NT>
+template <int MT, int RG, int XU, int DEPTH, bool NT, bool XRES>
 __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamArgs a) {
-    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage] then red[2][FRAGS][wave][64]
+    // XRES: [X blocks][XU KB] | [wave][DEPTH][RG*4 KB] | red;  else: [wave][DEPTH][(RG*4 + XU) KB] | red[2][FRAGS][wave][64]
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
 
-    constexpr int PER_STAGE = RG * 4 + XU;
+    constexpr int PER_STAGE = XRES ? RG * 4 : RG * 4 + XU;
     constexpr int STAGE_BYTES = PER_STAGE * 1024;
     constexpr int FRAGS = RG * MT;
     static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
@@ -220,9 +233,10 @@ __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamA
     const int src_row = q & 3;
     const int src_col = (q >> 2) * 64;
     const int rd_off = 1024 * (r >> 2) + 64 * (r & 3) + 16 * ((g - (r >> 2)) & 3);
-    const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
+    const int x_bytes = XRES ? blocks * XU * 1024 : 0;   // resident activations (needs m_tiles == 1)
+    const uint8_t* my_ring = ring + x_bytes + (size_t)wave * (DEPTH * STAGE_BYTES);
     const unsigned my_ring_lds = lds_addr(my_ring);
-    f32x4* red = reinterpret_cast<f32x4*>(ring + (size_t)waves * (DEPTH * STAGE_BYTES));
+    f32x4* red = reinterpret_cast<f32x4*>(ring + x_bytes + (size_t)waves * (DEPTH * STAGE_BYTES));
 
     auto tile_origin = [&](int j, int& m0, int& n0) {  // j-th tile of this workgroup
         const int t = (int)blockIdx.x + j * (int)gridDim.x;
@@ -247,11 +261,13 @@ __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamA
                 if (NT) dma_1kb_stream(src, slot + (rg * 4 + u) * 1024);
                 else dma_1kb(src, slot + (rg * 4 + u) * 1024);
             }
+        if (!XRES) {
 #pragma unroll
-        for (int u = 0; u < XU; u++) {
-            int row = m0 + 4 * u + src_row;
-            row = row < a.m ? row : a.m - 1;
-            dma_1kb(a.A + (size_t)row * a.k + koff + ((p + (u & 3)) & 3) * 16, slot + (RG * 4 + u) * 1024);
+            for (int u = 0; u < XU; u++) {
+                int row = m0 + 4 * u + src_row;
+                row = row < a.m ? row : a.m - 1;
+                dma_1kb(a.A + (size_t)row * a.k + koff + ((p + (u & 3)) & 3) * 16, slot + (RG * 4 + u) * 1024);
+            }
         }
     };
 
@@ -261,14 +277,17 @@ __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamA
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    int left_in_tile = per_tile;  // stages of the current tile not yet consumed
     auto consume = [&](int i) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
+        // activations: in the stage, or in the resident copy at this stage's K block
+        const uint8_t* xs = XRES ? ring + (size_t)(wave + (per_tile - left_in_tile) * waves) * (XU * 1024) + rd_off
+                                 : slot + RG * 4096;
 #pragma unroll
         for (int kc = 0; kc < 4; kc++) {
             i64x2 x[MT];
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-                x[mt] = *reinterpret_cast<const i64x2*>(slot + (RG * 4 + mt * 4) * 1024 + kc * 256);
+            for (int mt = 0; mt < MT; mt++) x[mt] = *reinterpret_cast<const i64x2*>(xs + mt * 4096 + kc * 256);
 #pragma unroll
             for (int rg = 0; rg < RG; rg++) {
                 const i64x2 w = *reinterpret_cast<const i64x2*>(slot + rg * 4096 + kc * 256);
@@ -307,13 +326,34 @@ __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamA
             for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     };
 
+    if (XRES) {
+        // K block kb of the activations is fetched by wave kb % waves; every wave then starts its
+        // weight ring, waits for its own share (older than the ring's DMAs) and meets the others
+        const unsigned x_lds = lds_addr(ring);
+        int x_issued = 0;
+        for (int kb = wave; kb < blocks; kb += waves) {
+#pragma unroll
+            for (int u = 0; u < XU; u++) {
+                int row = 4 * u + src_row;
+                row = row < a.m ? row : a.m - 1;
+                dma_1kb(a.A + (size_t)row * a.k + ((size_t)kb << 8) + src_col + ((p + (u & 3)) & 3) * 16,
+                        x_lds + (unsigned)(kb * XU + u) * 1024);
+            }
+            x_issued += XU;
+        }
+        (void)x_issued;
+    }
+
     if (per_tile == 0) {  // more waves than K blocks: this wave only takes part in the reductions
+        if (XRES) {
+            wait_vmcnt<0>();
+            __syncthreads();
+        }
         for (int j = 0; j < my_tiles; j++) tile_done(j);
         return;
     }
 
     // stage i ends a tile when it is this wave's last K block of that tile
-    int left_in_tile = per_tile;  // stages of the current tile not yet consumed
     int tile_j = 0;
     auto after_consume = [&]() {
         if (--left_in_tile == 0) {
@@ -325,6 +365,10 @@ __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamA
     if (total >= DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) issue(d);
+        if (XRES) {
+            wait_vmcnt_upto(DEPTH * PER_STAGE);   // this wave's activation blocks are older than its DEPTH stages
+            __syncthreads();
+        }
         int i = 0;
         for (; i + DEPTH < total; i++) {
             wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
@@ -342,6 +386,152 @@ __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamA
         drain_ring<0, DEPTH, PER_STAGE>(consume_and_close, i);
     } else {
         for (int i = 0; i < total; i++) issue(i);
+        wait_vmcnt<0>();
+        if (XRES) __syncthreads();
+        for (int i = 0; i < total; i++) {
+            consume(i);
+            after_consume();
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Wave-per-tile variant with the activations resident in LDS, for shapes with many tiles and a
+// short K (the MLP up-projection): every wave owns whole 16*RG-row tiles over the full K range,
+// so there is no cross-wave reduction and no barrier after the prologue.  The whole activation
+// matrix (ceil(m/4) KB per 256-byte K block) is fetched once per workgroup and shared by its
+// waves, which removes a third of the DMA instructions and of the L2 traffic at m = 8.  Wave
+// (workgroup b, wave w) walks tiles b*W + w, + total waves, ...; its weight ring runs across
+// tile boundaries.
+template <int MT, int RG, int XU, int DEPTH, bool NT>
+__global__ void __launch_bounds__(1024) lds_gemm_wavetile_kernel(const StreamArgs a) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // X[blocks][XU KB] | [wave][DEPTH][RG*4 KB]
+
+    constexpr int PER_STAGE = RG * 4;
+    constexpr int STAGE_BYTES = PER_STAGE * 1024;
+    constexpr int FRAGS = RG * MT;
+    static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
+    static_assert(MT == 1 || XU > 4, "two activation blocks need more than four DMA instructions");
+
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int waves = a.waves;
+    const int r = lane & 15, g = lane >> 4;
+
+    const int blocks = a.k >> 8;
+    const int total_tiles = a.n_tiles * a.m_tiles;
+    const int total_waves = (int)gridDim.x * waves;
+    const int gw = (int)blockIdx.x * waves + wave;
+    const int my_tiles = gw < total_tiles ? (total_tiles - gw + total_waves - 1) / total_waves : 0;
+    const int total = blocks * my_tiles;
+
+    const int q = lane >> 2, p = lane & 3;
+    const int src_row = q & 3;
+    const int src_col = (q >> 2) * 64;
+    const int rd_off = 1024 * (r >> 2) + 64 * (r & 3) + 16 * ((g - (r >> 2)) & 3);
+    const int x_bytes = blocks * XU * 1024;
+    const uint8_t* my_ring = ring + x_bytes + (size_t)wave * (DEPTH * STAGE_BYTES);
+    const unsigned my_ring_lds = lds_addr(my_ring);
+    const unsigned x_lds = lds_addr(ring);
+
+    // ---- resident activations: K block kb is fetched by wave kb % waves (m_tiles == 1) ----------
+    int x_issued = 0;
+    for (int kb = wave; kb < blocks; kb += waves) {
+#pragma unroll
+        for (int u = 0; u < XU; u++) {
+            int row = 4 * u + src_row;
+            row = row < a.m ? row : a.m - 1;
+            dma_1kb(a.A + (size_t)row * a.k + ((size_t)kb << 8) + src_col + ((p + (u & 3)) & 3) * 16,
+                    x_lds + (unsigned)(kb * XU + u) * 1024);
+        }
+        x_issued += XU;
+    }
+
+    auto issue = [&](int i) {
+        const int j = i / blocks;
+        const int kb = i - j * blocks;
+        const int n0 = ((gw + j * total_waves) % a.n_tiles) * (16 * RG);
+        const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
+        const size_t koff = ((size_t)kb << 8) + src_col;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                int row = n0 + rg * 16 + 4 * u + src_row;
+                row = row < a.n ? row : a.n - 1;
+                const uint8_t* src = a.B + (size_t)row * a.b_stride + koff + ((p + u) & 3) * 16;
+                if (NT) dma_1kb_stream(src, slot + (rg * 4 + u) * 1024);
+                else dma_1kb(src, slot + (rg * 4 + u) * 1024);
+            }
+    };
+
+    f32x4 acc[RG][MT];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    int kb_cur = 0;  // K block of the stage being consumed
+    auto consume = [&](int i) {
+        const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
+        const uint8_t* xs = ring + (size_t)kb_cur * (XU * 1024) + rd_off;
+#pragma unroll
+        for (int kc = 0; kc < 4; kc++) {
+            i64x2 x[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) x[mt] = *reinterpret_cast<const i64x2*>(xs + mt * 4096 + kc * 256);
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                const i64x2 w = *reinterpret_cast<const i64x2*>(slot + rg * 4096 + kc * 256);
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.x, x[mt].x, acc[rg][mt], 0, 0, 0);
+                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.y, x[mt].y, acc[rg][mt], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    const float scale = a.scale ? a.scale[0] : 1.0f;
+    int tile_j = 0;
+    auto after_consume = [&]() {
+        if (++kb_cur == blocks) {   // the tile is complete: scale, round, store, start the next one
+            kb_cur = 0;
+            const int n0 = ((gw + tile_j * total_waves) % a.n_tiles) * (16 * RG);
+            tile_j++;
+#pragma unroll
+            for (int f = 0; f < FRAGS; f++) {
+                store_fragment(a, acc[f / MT][f % MT], scale, (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g);
+                acc[f / MT][f % MT] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+    };
+
+    // weight prologue first, so that HBM is busy while the activations arrive from L2
+    const int pro = total < DEPTH ? total : DEPTH;
+    for (int d = 0; d < pro; d++) issue(d);
+    // this wave's share of the activations was issued before its weight stages: once at most
+    // pro * PER_STAGE DMAs are outstanding it has landed; the barrier publishes everyone's share
+    if (x_issued > 0) wait_vmcnt_upto(pro * PER_STAGE);
+    __syncthreads();
+
+    if (total >= DEPTH) {
+        int i = 0;
+        for (; i + DEPTH < total; i++) {
+            wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            consume(i);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            issue(i + DEPTH);
+            __builtin_amdgcn_sched_barrier(0);
+            after_consume();
+        }
+        auto consume_and_close = [&](int ii) {
+            consume(ii);
+            after_consume();
+        };
+        drain_ring<0, DEPTH, PER_STAGE>(consume_and_close, i);
+    } else {
         wait_vmcnt<0>();
         for (int i = 0; i < total; i++) {
             consume(i);

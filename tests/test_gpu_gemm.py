@@ -190,6 +190,15 @@ def test_lds_ring_persistent(sg, oracle, cfg, shape):
     assert sg.skinny_gemm_tuned(A, B, D2, S, **kw) == 0
     torch.cuda.synchronize()
     assert np.array_equal(bits(D2), got)
+    # ... and so does the variant that keeps the activations resident in LDS (one activation tile only)
+    if m <= (16 if m <= 16 else 32):
+        D3 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        kw.update(persistent_wgs_per_cu=per_cu, wave_tiles=2)
+        rc = sg.skinny_gemm_tuned(A, B, D3, S, **kw)
+        torch.cuda.synchronize()
+        if rc != 6:
+            assert rc == 0, sg.strerror(rc)
+            assert np.array_equal(bits(D3), got)
 
 
 RING_CONFIGS = [
@@ -297,6 +306,42 @@ def test_mid_batch_config4_shapes(sg, oracle, m, n, k):
     torch.cuda.synchronize()
     assert torch.equal(D2.float(), 2 * D.float())
     assert not torch.isnan(D.float()).any()
+
+
+WAVETILE_CONFIGS = [
+    # waves per workgroup, row_tiles, depth, workgroups per CU
+    (1, 1, 2, 1),
+    (7, 1, 3, 1),
+    (4, 2, 2, 2),
+    (3, 1, 8, 1),
+    (8, 1, 2, 4),
+    (2, 4, 3, 1),
+]
+
+
+@pytest.mark.parametrize("cfg", WAVETILE_CONFIGS)
+@pytest.mark.parametrize("shape", [(8, 28672, 1024), (1, 4096, 4096), (5, 9000, 768), (16, 6144, 2048), (32, 8192, 1024),
+                                   (3, 128, 512), (13, 2000, 256)])
+def test_lds_ring_wave_tiles(sg, oracle, cfg, shape):
+    """Every wave owns whole tiles over the full K range; activations resident in LDS."""
+    waves, row_tiles, depth, per_cu = cfg
+    m, n, k = shape
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=12)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kw = dict(engine=2, waves=waves, row_tiles=row_tiles, depth=depth, persistent_wgs_per_cu=per_cu, wave_tiles=1)
+    rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
+    torch.cuda.synchronize()
+    if rc == 6:
+        pytest.skip("configuration not compiled / does not fit LDS")
+    assert rc == 0, sg.strerror(rc)
+    got = bits(D)
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
+    D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_tuned(A, B, D2, S, **kw) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(D2), got)
 
 
 def test_torch_binding_surface(sg, oracle):
