@@ -29,6 +29,10 @@ SHAPES = {"qkv": (6144, 4096), "o": (4096, 4096), "gate_up": (28672, 4096), "dow
 M_SWEEP = (1, 2, 4, 8, 16, 32)
 HBM_PEAK_GBS = 8000.0
 COLD_BYTES = 640e6          # per shape: distinct weight bytes cycled through (> 2x the 256 MB cache)
+# HBM bytes per launch of the dominant kernel (gate_up, M = 8), measured off-line with two
+# rocprofv3 --pmc runs (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0, factors from a 256 MiB copy);
+# the runs and their arithmetic are in profiles/dense_gemm_decode_step_m8_pmc_traffic.md
+RECORDED_TRAFFIC = {("gate_up", 8): 118329364}
 
 
 def gemm_bytes(m, n, k):
@@ -44,6 +48,9 @@ def main():
     ap.add_argument("--m", type=int, default=8, help="activation rows of the timed step")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs (for counter runs)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run three 256 MiB device-to-device copies (known traffic, to scale profiler counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1")
@@ -104,19 +111,36 @@ def main():
         for i in range(args.warmup):
             step(i, st)
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        if args.no_graph:
             st = torch.cuda.current_stream().cuda_stream
+            t_host0 = time.perf_counter()
+            e0.record()
             for i in range(args.steps):
                 step(args.warmup + i, st)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t_host0 = time.perf_counter()
-        e0.record()
-        graph.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        t_host1 = time.perf_counter()
+            e1.record()
+            torch.cuda.synchronize()
+            t_host1 = time.perf_counter()
+        else:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                st = torch.cuda.current_stream().cuda_stream
+                for i in range(args.steps):
+                    step(args.warmup + i, st)
+            torch.cuda.synchronize()
+            t_host0 = time.perf_counter()
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            t_host1 = time.perf_counter()
+        if args.calibration_copy:
+            src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            del src, dst
     ms_total = e0.elapsed_time(e1)
     ms_per_step = ms_total / args.steps
     step_bytes = sum(gemm_bytes(args.m, *SHAPES[name]) for name in order)
@@ -140,6 +164,17 @@ def main():
 
     def back_to_back_us(name, m, reps):
         """Graph of `reps` launches on rotating buffers: time per launch including dispatch gaps."""
+        if args.no_graph:
+            with torch.cuda.stream(side):
+                st = torch.cuda.current_stream().cuda_stream
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                a.record()
+                for i in range(reps):
+                    launch(name, m, i, st)
+                b.record()
+                torch.cuda.synchronize()
+            return a.elapsed_time(b) * 1e3 / reps
         with torch.cuda.stream(side):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=side):
@@ -163,7 +198,7 @@ def main():
     dom_bytes = gemm_bytes(args.m, *SHAPES[dom])
     achieved = dom_bytes / (dom_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": RECORDED_TRAFFIC.get((dom, args.m)),
                 "kernel": "dense skinny GEMM, gate_up 28672x4096, M=%d" % args.m,
                 "bytes_per_launch": dom_bytes, "us_per_launch": round(dom_us, 3),
                 "us_per_launch_own_event_pair": round(dom_ev_mean_us, 3)}
