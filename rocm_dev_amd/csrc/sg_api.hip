@@ -372,11 +372,33 @@ static Config pick_config(int m, int n, int k, int cu_count) {
                 c.wavetile = 2;
                 return c;
             }
+            if (c.mt == 2) {                    // wide tiles share one activation stage among four weight tiles
+                c.persist = 0;
+                c.rg = 4;
+                c.waves = 1;
+                c.depth = 2;
+                return c;
+            }
             c.depth = 3;
             c.waves = 6;
             while (c.waves > 2 && (size_t)c.waves * (c.depth * (4 + xu0) + 2 * c.mt) * 1024 + 4096 > 159 * 1024)
                 c.waves--;
             if (c.waves == 5) c.waves = 4;
+        } else if (c.mt == 2) {                 // 17..32 activation rows: the activation traffic rivals the weights'
+            if (blocks >= 48) {
+                c.rg = 2;
+                c.waves = 2;
+                c.depth = 3;
+                c.split_k = 2;
+            } else if (tiles16 * 4 >= cu_count * 5) {
+                c.rg = 2;
+                c.waves = 2;
+                c.depth = 2;
+            } else {
+                c.rg = 1;
+                c.waves = 3;
+                c.depth = 2;
+            }
         } else {                                // about one tile per CU: few waves, deep rings
             c.rg = 1;
             c.waves = blocks >= 48 ? 2 : 1;

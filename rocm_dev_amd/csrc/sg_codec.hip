@@ -166,9 +166,11 @@ __global__ void __launch_bounds__(256) fp8_decode_rows_kernel(const uint8_t* __r
         o[j >> 1][2 * (j & 1)] = cvt_bf16x2(__fmul_rn(lo.x, s), __fmul_rn(lo.y, s));
         o[j >> 1][2 * (j & 1) + 1] = cvt_bf16x2(__fmul_rn(hi.x, s), __fmul_rn(hi.y, s));
     }
+    // plain stores: with 32 bytes per lane the non-temporal hint costs a third of the bandwidth
+    // (measured 3.9 vs 6.0 TB/s for this 1-read : 2-write pattern)
     u32x4* y = reinterpret_cast<u32x4*>(Y) + 2 * idx;
-    __builtin_nontemporal_store(o[0], y);
-    __builtin_nontemporal_store(o[1], y + 1);
+    y[0] = o[0];
+    y[1] = o[1];
 }
 
 template <int NBUF>
@@ -216,9 +218,11 @@ __global__ void __launch_bounds__(256) fp8_reduce_rows_kernel(const uint8_t* __r
     u32x4 o[2];
 #pragma unroll
     for (int j = 0; j < 8; j++) o[j >> 2][j & 3] = cvt_bf16x2(acc[2 * j], acc[2 * j + 1]);
+    // plain stores: with 32 bytes per lane the non-temporal hint costs a third of the bandwidth
+    // (measured 3.9 vs 6.0 TB/s for this 1-read : 2-write pattern)
     u32x4* y = reinterpret_cast<u32x4*>(Y) + 2 * idx;
-    __builtin_nontemporal_store(o[0], y);
-    __builtin_nontemporal_store(o[1], y + 1);
+    y[0] = o[0];
+    y[1] = o[1];
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
