@@ -259,8 +259,8 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
         a.ws = w->partials;
         a.counters = w->counters;
     }
-    const size_t lds = (size_t)c.depth * (bn + bm) * 128;
-    if (lds > 159 * 1024) return SG_INVALID_CONFIG;
+    const size_t lds = (size_t)c.depth * (bn + bm) * 128 + (c.split_k > 1 ? 16 : 0);
+    if (lds > 160 * 1024) return SG_INVALID_CONFIG;
     return launch_mid(c.rg, c.mt, c.depth, a, (unsigned)(tiles * c.split_k), lds, stream);
 }
 

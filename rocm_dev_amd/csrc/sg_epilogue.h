@@ -33,6 +33,11 @@ struct StreamArgs {
 
 // Writes one finished 16(n) x 16(m) fragment: lane owns m = m_base + l%16, n = n_base + 4*(l/16)..+3.
 __device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, float scale, int m_idx, int n_idx) {
+    // Pin the fragment before the lane-divergent exit below.  An MFMA needs every lane of the wave
+    // (it reads all lanes' operand registers), but the compiler is free to sink the loads and the
+    // MFMA that produce `v` into the region where only lanes with m_idx < m are active - it did so
+    // with the 16x16x128 instruction - and the operand rows supplied by the masked lanes are then garbage.
+    asm volatile("" : "+v"(v));
     if (m_idx >= a.m) return;
     v *= scale;
     const size_t off = (size_t)m_idx * a.n + n_idx;

@@ -73,6 +73,39 @@ __device__ __forceinline__ void drain_ring(Consume& consume, int i) {
     if constexpr (D + 1 < DEPTH) drain_ring<D + 1, DEPTH, PER_STAGE>(consume, i);
 }
 
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+
+// One 256-byte K block of a stage: weights at w (16*RG rows, 4 KB per 16-row tile), activations
+// at x (4 KB per 16-row block), both already offset by the lane's read offset.  The four 64-byte
+// chunks of the block feed two v_mfma_scale_f32_16x16x128_f8f6f4 (unit scales): lane (r, g)
+// supplies its 16-byte pieces of chunks 0,1 to the first and of chunks 2,3 to the second - the
+// same pieces for both operands, so the K permutation cancels.  The 128-wide instruction runs at
+// the full FP8 rate of gfx950 (measured 4.9 PFLOP/s against 0.8-1.3 for v_mfma_f32_16x16x32_fp8_fp8).
+template <int MT, int RG>
+__device__ __forceinline__ void mma_block_256(const uint8_t* w, const uint8_t* x, f32x4 (&acc)[RG][MT]) {
+    i32x8 xv[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(x + mt * 4096 + (2 * h) * 256);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(x + mt * 4096 + (2 * h + 1) * 256);
+            xv[mt][h] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(w + rg * 4096 + (2 * h) * 256);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(w + rg * 4096 + (2 * h + 1) * 256);
+            const i32x8 wv = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+                acc[rg][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, xv[mt][h], acc[rg][mt], 0, 0, 0, 0x7f7f7f7f, 0,
+                                                                               0x7f7f7f7f);
+        }
+}
+
 constexpr int lds_stage_bytes(int RG, int XU) { return (RG * 4 + XU) * 1024; }
 
 // XU = activation DMA instructions per stage (4 rows each): ceil(min(m, 16*MT) / 4)
@@ -155,22 +188,7 @@ __global__ void __launch_bounds__(1024) lds_gemm_kernel(const StreamArgs a) {
 
     auto consume = [&](int i) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
-#pragma unroll
-        for (int kc = 0; kc < 4; kc++) {
-            i64x2 x[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++)
-                x[mt] = *reinterpret_cast<const i64x2*>(slot + (RG * 4 + mt * 4) * 1024 + kc * 256);
-#pragma unroll
-            for (int rg = 0; rg < RG; rg++) {
-                const i64x2 w = *reinterpret_cast<const i64x2*>(slot + rg * 4096 + kc * 256);
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.x, x[mt].x, acc[rg][mt], 0, 0, 0);
-                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.y, x[mt].y, acc[rg][mt], 0, 0, 0);
-                }
-            }
-        }
+        mma_block_256<MT, RG>(slot, slot + RG * 4096, acc);
     };
 
     if (mine >= DEPTH) {
@@ -283,21 +301,7 @@ __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamA
         // activations: in the stage, or in the resident copy at this stage's K block
         const uint8_t* xs = XRES ? ring + (size_t)(wave + (per_tile - left_in_tile) * waves) * (XU * 1024) + rd_off
                                  : slot + RG * 4096;
-#pragma unroll
-        for (int kc = 0; kc < 4; kc++) {
-            i64x2 x[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++) x[mt] = *reinterpret_cast<const i64x2*>(xs + mt * 4096 + kc * 256);
-#pragma unroll
-            for (int rg = 0; rg < RG; rg++) {
-                const i64x2 w = *reinterpret_cast<const i64x2*>(slot + rg * 4096 + kc * 256);
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.x, x[mt].x, acc[rg][mt], 0, 0, 0);
-                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.y, x[mt].y, acc[rg][mt], 0, 0, 0);
-                }
-            }
-        }
+        mma_block_256<MT, RG>(slot, xs, acc);
     };
 
     const float scale = a.scale ? a.scale[0] : 1.0f;
@@ -474,22 +478,7 @@ __global__ void __launch_bounds__(1024) lds_gemm_wavetile_kernel(const StreamArg
     int kb_cur = 0;  // K block of the stage being consumed
     auto consume = [&](int i) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
-        const uint8_t* xs = ring + (size_t)kb_cur * (XU * 1024) + rd_off;
-#pragma unroll
-        for (int kc = 0; kc < 4; kc++) {
-            i64x2 x[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++) x[mt] = *reinterpret_cast<const i64x2*>(xs + mt * 4096 + kc * 256);
-#pragma unroll
-            for (int rg = 0; rg < RG; rg++) {
-                const i64x2 w = *reinterpret_cast<const i64x2*>(slot + rg * 4096 + kc * 256);
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.x, x[mt].x, acc[rg][mt], 0, 0, 0);
-                    acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w.y, x[mt].y, acc[rg][mt], 0, 0, 0);
-                }
-            }
-        }
+        mma_block_256<MT, RG>(slot, ring + (size_t)kb_cur * (XU * 1024) + rd_off, acc);
     };
 
     const float scale = a.scale ? a.scale[0] : 1.0f;

@@ -32,14 +32,13 @@
 
 namespace sg {
 
-typedef int i32x8 __attribute__((ext_vector_type(8)));
-
 // RGW: 16-row weight fragments per wave (2 or 4)  -> BN = 32*RGW rows per workgroup
 // MH : 16-row activation fragments per wave (2, 4, 8) -> up to 32*MH activation rows per tile
 template <int RGW, int MH, int DEPTH>
 __global__ void __launch_bounds__(256) mid_gemm_kernel(const StreamArgs a) {
-    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [DEPTH][W rows | X rows][128]
-    __shared__ unsigned arrival;
+    // [DEPTH][W rows | X rows][128], then (split-K only) 16 bytes for the arrival broadcast; no static
+    // LDS, so that two workgroups of exactly half the CU's LDS can share a CU
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
 
     constexpr int BN = 32 * RGW;
     constexpr int BM = 32 * MH;
@@ -178,10 +177,11 @@ __global__ void __launch_bounds__(256) mid_gemm_kernel(const StreamArgs a) {
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    volatile unsigned* arrival = reinterpret_cast<volatile unsigned*>(ring + (size_t)DEPTH * STAGE_BYTES);
     if (threadIdx.x == 0)
-        arrival = __hip_atomic_fetch_add(&a.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *arrival = __hip_atomic_fetch_add(&a.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (arrival != (unsigned)(a.split_k - 1)) return;
+    if (*arrival != (unsigned)(a.split_k - 1)) return;
     store_all([&](int rg, int mb) {
         const float* p = ws_tile + (size_t)wave * (RGW * MH * 256) + (rg * MH + mb) * 256 + lane;
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
