@@ -240,8 +240,11 @@ static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
 static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) {
     if (a.k % 128 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if ((c.rg != 2 && c.rg != 4) || (c.mt != 2 && c.mt != 4 && c.mt != 8) || c.depth < 2) return SG_INVALID_CONFIG;
-    const int bn = 32 * c.rg, bm = 32 * c.mt;
-    a.waves = 4;
+    const int wn = c.waves == 8 ? 4 : 2;          // 8 waves = 4 (N) x 2 (M), otherwise 2 x 2
+    if (c.waves != 4 && c.waves != 8) return SG_INVALID_CONFIG;
+    const int bn = 16 * c.rg * wn, bm = 32 * c.mt;
+    if (bn % (16 * wn) != 0 || bm % (16 * wn) != 0) return SG_INVALID_CONFIG;
+    a.waves = c.waves;
     a.split_k = c.split_k;
     a.n_tiles = (a.n + bn - 1) / bn;
     a.m_tiles = (a.m + bm - 1) / bm;
@@ -254,35 +257,69 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
     if (c.split_k > 1) {
         Workspace* w;
         if (int rc = get_workspace(&w)) return rc;
-        const size_t per_tile = (size_t)4 * c.rg * c.mt * 1024;   // fp32 fragments of one workgroup tile
+        const size_t per_tile = (size_t)c.waves * c.rg * c.mt * 1024;   // fp32 fragments of one workgroup tile
         if (tiles > w->n_counters || tiles * c.split_k * per_tile > w->partial_bytes) return SG_WORKSPACE_TOO_SMALL;
         a.ws = w->partials;
         a.counters = w->counters;
     }
     const size_t lds = (size_t)c.depth * (bn + bm) * 128 + (c.split_k > 1 ? 16 : 0);
     if (lds > 160 * 1024) return SG_INVALID_CONFIG;
-    return launch_mid(c.rg, c.mt, c.depth, a, (unsigned)(tiles * c.split_k), lds, stream);
+    return launch_mid(c.rg, c.mt, c.depth, wn, a, (unsigned)(tiles * c.split_k), lds, stream);
 }
 
+// Mid-batch heuristic, fitted to timings of the Llama-3-70B projection shapes at M = 64..256:
+// what matters first is that one round of workgroups covers the device (a second, partly
+// filled round costs more than any tile-shape effect), then that the round is as full as
+// possible, then the tile: 128x128 and 128x64 tiles on eight waves beat both smaller tiles
+// (more operand traffic per flop) and 256-wide ones (one workgroup per CU and a two-slot ring),
+// which only pay off when nothing else fits in one round.  K may be split up to four ways as
+// long as every split keeps 32 K blocks.
 static Config pick_mid(int m, int n, int k, int cu_count) {
-    Config c;
+    struct Tile { int bn, bm, waves; };
+    static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4},
+                                 {256, 128, 8}, {256, 64, 8}, {128, 256, 8}, {256, 256, 8}};
+    const int bm_max = m <= 64 ? 64 : (m <= 128 ? 128 : 256);
+    const int blocks = k / 128;
+    Config best;
+    long best_rounds = -1, best_wgs = 0;
+    for (const Tile& t : order) {
+        if (t.bm > bm_max) continue;
+        const long tiles = (long)((n + t.bn - 1) / t.bn) * ((m + t.bm - 1) / t.bm);
+        for (int sk = 1; sk <= 4; sk *= 2) {
+            if (sk > 1 && blocks / sk < 32) break;
+            const long wgs = tiles * sk;
+            const long rounds = (wgs + cu_count - 1) / cu_count;
+            const bool better = best_rounds < 0 || rounds < best_rounds ||
+                                (rounds == best_rounds && wgs * 16 > best_wgs * 17) ||   // clearly fuller round
+                                // as full with less splitting, when the splits had become short
+                                (rounds == best_rounds && wgs == best_wgs && sk < best.split_k &&
+                                 blocks / best.split_k < 48);
+            if (!better) continue;
+            best_rounds = rounds;
+            best_wgs = wgs;
+            best.waves = t.waves;
+            best.rg = t.bn / (t.waves * 8);      // 16-row tiles per wave: bn = 16 * rg * (waves / 2)
+            best.mt = t.bm / 32;
+            best.split_k = sk;
+        }
+    }
+    Config c = best;
+    bool co_resident = false;
+    if (m <= 64 && (long)((n + 127) / 128) * 2 >= 3L * cu_count) {
+        // memory-bound and many tiles: several small two-slot workgroups per CU hide the DMA
+        // latency better than one deep ring
+        c.waves = 8; c.rg = 2; c.mt = 2; c.split_k = 1;
+        co_resident = true;
+    }
     c.engine = ENGINE_MID;
     c.nt = 1;
     c.persist = 0;
     c.wavetile = 0;
     c.ku = 2;
-    c.waves = 4;
-    c.mt = m <= 64 ? 2 : (m <= 128 ? 4 : 8);
-    c.rg = (n + 127) / 128 >= cu_count / 2 ? 4 : 2;
-    const int tiles = (n + 32 * c.rg - 1) / (32 * c.rg) * ((m + 32 * c.mt - 1) / (32 * c.mt));
-    const int blocks = k / 128;
-    c.split_k = 1;
-    // few tiles: split K until every CU has a workgroup, keeping at least 16 K blocks per split
-    while (tiles * c.split_k * 2 <= cu_count && blocks / (c.split_k * 2) >= 16 && c.split_k < 8) c.split_k *= 2;
-    c.depth = 6;
-    while (c.depth > 2 && ((size_t)c.depth * (32 * c.rg + 32 * c.mt) * 128 > 159 * 1024 ||
-                           (c.depth - 2) * (c.rg + c.mt) > 63 || c.depth == 5))
-        c.depth--;
+    const int bn = 8 * c.rg * c.waves, bm = 32 * c.mt;
+    const int per_wave = (bn + bm) / (8 * c.waves);   // DMA instructions per wave and stage
+    c.depth = co_resident ? 2 : 4;
+    while (c.depth > 2 && ((size_t)c.depth * (bn + bm) * 128 > 159 * 1024 || (c.depth - 2) * per_wave > 63)) c.depth--;
     return c;
 }
 

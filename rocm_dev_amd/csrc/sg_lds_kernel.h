@@ -107,10 +107,13 @@ __device__ __forceinline__ void mma_block_256(const uint8_t* w, const uint8_t* x
 }
 
 constexpr int lds_stage_bytes(int RG, int XU) { return (RG * 4 + XU) * 1024; }
+// Eight or more accumulator fragments per wave need more than the 128 VGPRs a 16-wave workgroup
+// leaves each wave; those instantiations accept at most 8 waves per workgroup.
+constexpr int lds_launch_bound(int MT, int RG) { return RG * MT >= 8 ? 512 : 1024; }
 
 // XU = activation DMA instructions per stage (4 rows each): ceil(min(m, 16*MT) / 4)
 template <int MT, int RG, int XU, int DEPTH, bool NT>
-__global__ void __launch_bounds__(1024) lds_gemm_kernel(const StreamArgs a) {
+__global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
     __shared__ unsigned arrival;
 
@@ -227,7 +230,7 @@ __global__ void __launch_bounds__(1024) lds_gemm_kernel(const StreamArgs a) {
 // The reduction scratch is double-buffered by tile parity, which leaves one barrier per tile.
 // No cross-workgroup split-K in this variant.
 template <int MT, int RG, int XU, int DEPTH, bool NT, bool XRES>
-__global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamArgs a) {
+__global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_kernel(const StreamArgs a) {
     // XRES: [X blocks][XU KB] | [wave][DEPTH][RG*4 KB] | red;  else: [wave][DEPTH][(RG*4 + XU) KB] | red[2][FRAGS][wave][64]
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
 
@@ -408,7 +411,7 @@ __global__ void __launch_bounds__(1024) lds_gemm_persistent_kernel(const StreamA
 // (workgroup b, wave w) walks tiles b*W + w, + total waves, ...; its weight ring runs across
 // tile boundaries.
 template <int MT, int RG, int XU, int DEPTH, bool NT>
-__global__ void __launch_bounds__(1024) lds_gemm_wavetile_kernel(const StreamArgs a) {
+__global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_wavetile_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // X[blocks][XU KB] | [wave][DEPTH][RG*4 KB]
 
     constexpr int PER_STAGE = RG * 4;

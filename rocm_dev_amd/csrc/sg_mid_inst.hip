@@ -5,9 +5,9 @@
 
 namespace sg {
 
-template <int RGW, int MH, int DEPTH>
+template <int RGW, int MH, int DEPTH, int WN>
 static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
-    auto kernel = mid_gemm_kernel<RGW, MH, DEPTH>;
+    auto kernel = mid_gemm_kernel<RGW, MH, DEPTH, WN>;
     static size_t attr_bytes[16] = {};
     if (lds > 48 * 1024) {
         int dev = 0;
@@ -22,19 +22,23 @@ static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_
             attr_bytes[dev] = lds;
         }
     }
-    kernel<<<dim3(grid), dim3(256), lds, stream>>>(a);
+    kernel<<<dim3(grid), dim3(WN * 128), lds, stream>>>(a);
     return report_hip("mid_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }
 
-#define SG_CASE(RGW_, MH_, DEPTH_)                                                     \
-    if (rgw == RGW_ && mh == MH_ && depth == DEPTH_) {                                 \
-        if constexpr ((DEPTH_ - 2) * (RGW_ + MH_) <= 63)                               \
-            return launch_one<RGW_, MH_, DEPTH_>(a, grid, lds, stream);                \
-        else                                                                           \
-            return SG_INVALID_CONFIG;                                                  \
+#define SG_CASE(RGW_, MH_, DEPTH_)                                                             \
+    if (rgw == RGW_ && mh == MH_ && depth == DEPTH_) {                                         \
+        if (wn == 2) {                                                                         \
+            if constexpr ((DEPTH_ - 2) * (RGW_ + MH_) <= 63)                                   \
+                return launch_one<RGW_, MH_, DEPTH_, 2>(a, grid, lds, stream);                 \
+            else                                                                               \
+                return SG_INVALID_CONFIG;                                                      \
+        }                                                                                      \
+        if (wn == 4) return launch_one<RGW_, MH_, DEPTH_, 4>(a, grid, lds, stream);            \
+        return SG_INVALID_CONFIG;                                                              \
     }
 
-int launch_mid(int rgw, int mh, int depth, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
+int launch_mid(int rgw, int mh, int depth, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
     SG_CASE(2, 2, 2) SG_CASE(2, 2, 3) SG_CASE(2, 2, 4) SG_CASE(2, 2, 6)
     SG_CASE(2, 4, 2) SG_CASE(2, 4, 3) SG_CASE(2, 4, 4) SG_CASE(2, 4, 6)
     SG_CASE(2, 8, 2) SG_CASE(2, 8, 3) SG_CASE(2, 8, 4)

@@ -34,23 +34,26 @@ namespace sg {
 
 // RGW: 16-row weight fragments per wave (2 or 4)  -> BN = 32*RGW rows per workgroup
 // MH : 16-row activation fragments per wave (2, 4, 8) -> up to 32*MH activation rows per tile
-template <int RGW, int MH, int DEPTH>
-__global__ void __launch_bounds__(256) mid_gemm_kernel(const StreamArgs a) {
+// WN : waves along N (2 or 4); the workgroup has WN x 2 waves
+template <int RGW, int MH, int DEPTH, int WN>
+__global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) {
     // [DEPTH][W rows | X rows][128], then (split-K only) 16 bytes for the arrival broadcast; no static
     // LDS, so that two workgroups of exactly half the CU's LDS can share a CU
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
 
-    constexpr int BN = 32 * RGW;
+    constexpr int WAVES = 2 * WN;
+    constexpr int BN = 16 * RGW * WN;
     constexpr int BM = 32 * MH;
-    constexpr int W_INSTR = BN / 8 / 4;   // DMA instructions per wave per stage for the weights
-    constexpr int X_INSTR = BM / 8 / 4;   // ... and for the activations
+    constexpr int W_INSTR = BN / 8 / WAVES;   // DMA instructions per wave per stage for the weights
+    constexpr int X_INSTR = BM / 8 / WAVES;   // ... and for the activations
+    static_assert(BN % (8 * WAVES) == 0 && BM % (8 * WAVES) == 0, "stage rows must split evenly over the waves' DMA instructions");
     constexpr int PER_STAGE = W_INSTR + X_INSTR;
     constexpr int STAGE_BYTES = (BN + BM) * 128;
     static_assert(DEPTH >= 2 && (DEPTH - 2) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
 
     const int lane = lane_id();
     const int wave = wave_id();
-    const int wn = wave & 1, wm = wave >> 1;
+    const int wn = wave % WN, wm = wave / WN;
 
     int bid = blockIdx.x;
     const int tile_n = bid % a.n_tiles;
@@ -73,14 +76,14 @@ __global__ void __launch_bounds__(256) mid_gemm_kernel(const StreamArgs a) {
     const uint8_t* xsrc[X_INSTR];
 #pragma unroll
     for (int i = 0; i < W_INSTR; i++) {
-        const int row_l = 8 * (4 * i + wave) + d_row;           // row inside the weight part of the stage
+        const int row_l = 8 * (WAVES * i + wave) + d_row;       // row inside the weight part of the stage
         int row = n0 + row_l;
         row = row < a.n ? row : a.n - 1;
         wsrc[i] = a.B + (size_t)row * a.b_stride + ((d_pp ^ ((row_l >> 1) & 7)) << 4);
     }
 #pragma unroll
     for (int i = 0; i < X_INSTR; i++) {
-        const int row_l = 8 * (4 * i + wave) + d_row;
+        const int row_l = 8 * (WAVES * i + wave) + d_row;
         int row = m0 + row_l;
         row = row < a.m ? row : a.m - 1;
         xsrc[i] = a.A + (size_t)row * a.k + ((d_pp ^ ((row_l >> 1) & 7)) << 4);
@@ -90,9 +93,9 @@ __global__ void __launch_bounds__(256) mid_gemm_kernel(const StreamArgs a) {
         const size_t koff = (size_t)(b_begin + s) << 7;
         const unsigned slot = ring_lds + (unsigned)(s % DEPTH) * STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < W_INSTR; i++) dma_1kb_stream(wsrc[i] + koff, slot + (4 * i + wave) * 1024);
+        for (int i = 0; i < W_INSTR; i++) dma_1kb_stream(wsrc[i] + koff, slot + (WAVES * i + wave) * 1024);
 #pragma unroll
-        for (int i = 0; i < X_INSTR; i++) dma_1kb(xsrc[i] + koff, slot + BN * 128 + (4 * i + wave) * 1024);
+        for (int i = 0; i < X_INSTR; i++) dma_1kb(xsrc[i] + koff, slot + BN * 128 + (WAVES * i + wave) * 1024);
     };
 
     // ---- LDS read offsets: lane (r, g) reads pieces 2g and 2g+1 of row r of a 16-row fragment --
@@ -161,7 +164,7 @@ __global__ void __launch_bounds__(256) mid_gemm_kernel(const StreamArgs a) {
     }
 
     // split-K: agent-scope partial stores, arrival counter, last workgroup sums in split order
-    constexpr int FRAGS_WG = 4 * RGW * MH;   // fragments of one workgroup tile
+    constexpr int FRAGS_WG = WAVES * RGW * MH;   // fragments of one workgroup tile
     const int tile_id = tile_m * a.n_tiles + tile_n;
     float* ws_tile = a.ws + ((size_t)tile_id * a.split_k) * (FRAGS_WG * 256);
     {

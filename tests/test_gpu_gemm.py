@@ -243,14 +243,20 @@ def test_producer_consumer_ring(sg, oracle, cfg, shape):
 
 
 MID_CONFIGS = [
-    # row_tiles (RGW), m_blocks (MH), depth, split_k
-    (2, 2, 2, 1),
-    (4, 2, 6, 1),
-    (2, 4, 3, 2),
-    (4, 4, 4, 1),
-    (2, 8, 3, 1),
-    (4, 8, 3, 4),
-    (4, 8, 2, 1),
+    # row_tiles (RGW), m_blocks (MH), depth, split_k, waves
+    (2, 2, 2, 1, 4),
+    (4, 2, 6, 1, 4),
+    (2, 4, 3, 2, 4),
+    (4, 4, 4, 1, 4),
+    (2, 8, 3, 1, 4),
+    (4, 8, 3, 4, 4),
+    (4, 8, 2, 1, 4),
+    (2, 2, 4, 1, 8),
+    (2, 4, 4, 2, 8),
+    (4, 4, 3, 1, 8),
+    (2, 8, 3, 4, 8),
+    (4, 8, 2, 1, 8),
+    (4, 2, 6, 2, 8),
 ]
 
 
@@ -258,14 +264,14 @@ MID_CONFIGS = [
 @pytest.mark.parametrize("shape", [(64, 512, 1024), (40, 130, 2048), (128, 1024, 2048), (256, 640, 4096), (200, 256, 4096),
                                    (300, 128, 1536), (33, 64, 128)])
 def test_mid_batch_engine(sg, oracle, cfg, shape):
-    """32 < m: weights streamed once, 2 x 2 waves per tile, 16x16x128 scaled MFMA with unit scales."""
-    rgw, mh, depth, split_k = cfg
+    """32 < m: weights streamed once, 2 x 2 or 4 x 2 waves per tile, 16x16x128 scaled MFMA with unit scales."""
+    rgw, mh, depth, split_k, waves = cfg
     m, n, k = shape
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=11)
     ref = oracle.gemm_omp(a8, b8, scale)
     A, B, S = dev(a8), dev(b8), scale_tensor(scale)
     D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
-    kw = dict(engine=4, split_k=split_k, row_tiles=rgw, m_blocks=mh, depth=depth)
+    kw = dict(engine=4, split_k=split_k, waves=waves, row_tiles=rgw, m_blocks=mh, depth=depth)
     rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
     torch.cuda.synchronize()
     if rc == 6:
@@ -279,7 +285,8 @@ def test_mid_batch_engine(sg, oracle, cfg, shape):
     assert np.array_equal(bits(D2), got)
 
 
-@pytest.mark.parametrize("m,n,k", [(64, 10240, 8192), (256, 8192, 8192), (128, 57344, 8192), (256, 8192, 28672)])
+@pytest.mark.parametrize("m,n,k", [(64, 10240, 8192), (128, 10240, 8192), (128, 8192, 8192), (256, 8192, 8192),
+                                   (128, 57344, 8192), (256, 57344, 8192), (64, 8192, 28672), (256, 8192, 28672)])
 def test_mid_batch_config4_shapes(sg, oracle, m, n, k):
     """BASELINE config 4 shapes at full size through the fastpath.  The oracle checks two
     512-row slices of the weight matrix (tiles are independent along n); the rest is covered
