@@ -97,7 +97,7 @@ struct Config {
     int split_k;  // workgroups per tile, splitting K among themselves
     int nt;       // weights loaded with the non-temporal hint
     int persist;  // LDS engine: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU walking the tiles
-    int wavetile; // LDS engine: 1 = every wave owns whole tiles, activations resident in LDS (persist = workgroups per CU);
+    int wavetile; // LDS engine, bits 0-1: 1 = every wave owns whole tiles, activations resident in LDS (persist = workgroups per CU);
                   //             2 = persistent K-split workgroups with the activations resident in LDS
 };
 
@@ -153,7 +153,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     // + 4 KB: lanes of activation rows that are not loaded read past the last slot
     size_t lds = (size_t)c.waves * c.depth * stage + 4096;
     unsigned grid = (unsigned)(tiles * c.split_k);
-    int mode = 0;
+    int mode = 0, extra_wave = 0;
     if (c.wavetile == 1) {
         // whole activation matrix resident: one tile row of activations only, no K split
         if (c.split_k != 1 || a.m_tiles != 1 || c.persist < 1) return SG_INVALID_CONFIG;
@@ -168,7 +168,8 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     } else if (c.persist > 0) {
         if (c.split_k != 1) return SG_INVALID_CONFIG;
         mode = 1;
-        if (c.wavetile == 2) {   // activations resident: stages hold weights only
+        if (c.wavetile & 4) extra_wave = 1;   // dedicated epilogue wave
+        if ((c.wavetile & 3) == 2) {   // activations resident: stages hold weights only
             if (a.m_tiles != 1) return SG_INVALID_CONFIG;
             mode = 3;
             lds = (size_t)(a.k / 256) * xu * 1024 + (size_t)c.waves * c.depth * c.rg * 4096 + 4096;
@@ -180,7 +181,8 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         if (want < grid) grid = (unsigned)want;
     }
     if (lds > 159 * 1024) return SG_INVALID_CONFIG;  // 160 KB per CU, minus the kernel's static LDS
-    const unsigned threads = (unsigned)c.waves * 64;
+    const unsigned threads = (unsigned)(c.waves + extra_wave) * 64;
+    if (threads > 1024) return SG_TOO_MANY_WARPS;
 #define SG_GO(MT, RG)                                                                                          \
     if (c.mt == MT && c.rg == RG)                                                                              \
         return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, mode, a, grid, threads, lds, stream);
@@ -403,12 +405,13 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             c.rg = 1;
             c.persist = 1;
             const size_t x_res = (size_t)blocks * xu0 * 1024;
-            c.waves = m <= 8 ? 8 : 6;
+            c.waves = m <= 8 ? 8 : 7;
             c.depth = 2;
             if (m <= 16 * c.mt && x_res + (size_t)c.waves * (c.depth * 4 + 2 * c.mt) * 1024 + 4096 <= 159 * 1024) {
-                c.wavetile = 2;
+                c.wavetile = 2 | 4;   // resident activations + a dedicated epilogue wave (0.3-0.9 us on gate_up)
                 return c;
             }
+            c.waves = m <= 8 ? 8 : 6;
             if (c.mt == 2) {                    // wide tiles share one activation stage among four weight tiles
                 c.persist = 0;
                 c.rg = 4;

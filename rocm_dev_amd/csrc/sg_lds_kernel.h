@@ -247,7 +247,12 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
     const int total_tiles = a.n_tiles * a.m_tiles;
     const int my_tiles = ((int)blockIdx.x < total_tiles) ? (total_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
     const int blocks = a.k >> 8;
-    const int per_tile = wave < blocks ? (blocks - wave + waves - 1) / waves : 0;
+    // a workgroup launched with one wave more than a.waves has a dedicated epilogue wave: it
+    // streams nothing and does every reduction and store, so that the streaming waves never have
+    // a store in their vmcnt queue (a store younger than the ring's DMAs makes every later
+    // vmcnt(n) wait for one DMA more than needed until the store is acknowledged)
+    const bool epilogue_wave = blockDim.x > (unsigned)waves * 64;
+    const int per_tile = (wave < waves && wave < blocks) ? (blocks - wave + waves - 1) / waves : 0;
     const int total = per_tile * my_tiles;
 
     const int q = lane >> 2, p = lane & 3;
@@ -312,16 +317,26 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
     auto tile_done = [&](int j) {
         int m0, n0;
         tile_origin(j, m0, n0);
-        if (waves == 1) {
+        if (waves == 1 && !epilogue_wave) {
 #pragma unroll
             for (int f = 0; f < FRAGS; f++)
                 store_fragment(a, acc[f / MT][f % MT], scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g);
         } else {
             f32x4* buf = red + (size_t)(j & 1) * (FRAGS * waves * 64);
+            if (wave < waves) {
 #pragma unroll
-            for (int f = 0; f < FRAGS; f++) buf[(f * waves + wave) * 64 + lane] = acc[f / MT][f % MT];
+                for (int f = 0; f < FRAGS; f++) buf[(f * waves + wave) * 64 + lane] = acc[f / MT][f % MT];
+            }
             __syncthreads();
-            for (int f = wave; f < FRAGS; f += waves) {
+            // without an epilogue wave the reducing wave rotates with the tile, so that the cost is
+            // spread over the waves
+            int first = wave - j % waves, step = waves;
+            first = first < 0 ? first + waves : first;
+            if (epilogue_wave) {
+                first = wave == waves ? 0 : FRAGS;
+                step = 1;
+            }
+            for (int f = first; f < FRAGS; f += step) {
                 f32x4 v = buf[(f * waves) * 64 + lane];
                 for (int w = 1; w < waves; w++) v += buf[(f * waves + w) * 64 + lane];
                 store_fragment(a, v, scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g);
@@ -338,7 +353,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
         // weight ring, waits for its own share (older than the ring's DMAs) and meets the others
         const unsigned x_lds = lds_addr(ring);
         int x_issued = 0;
-        for (int kb = wave; kb < blocks; kb += waves) {
+        for (int kb = wave < waves ? wave : blocks; kb < blocks; kb += waves) {
 #pragma unroll
             for (int u = 0; u < XU; u++) {
                 int row = 4 * u + src_row;

@@ -199,6 +199,17 @@ def test_lds_ring_persistent(sg, oracle, cfg, shape):
         if rc != 6:
             assert rc == 0, sg.strerror(rc)
             assert np.array_equal(bits(D3), got)
+    # ... and the variants with a dedicated epilogue wave (same partials, same order)
+    for wave_tiles in (4, 6):
+        if wave_tiles == 6 and m > (16 if m <= 16 else 32):
+            continue
+        D4 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        kw.update(persistent_wgs_per_cu=per_cu, wave_tiles=wave_tiles)
+        rc = sg.skinny_gemm_tuned(A, B, D4, S, **kw)
+        torch.cuda.synchronize()
+        if rc not in (4, 6):
+            assert rc == 0, sg.strerror(rc)
+            assert np.array_equal(bits(D4), got)
 
 
 RING_CONFIGS = [
