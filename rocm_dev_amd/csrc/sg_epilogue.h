@@ -76,7 +76,7 @@ __device__ __forceinline__ void finish_tile(const StreamArgs& a, f32x4 (&acc)[RG
     const int tile_id = tile_m * a.n_tiles + tile_n;
     float* ws_tile = a.ws + ((size_t)tile_id * a.split_k) * (FRAGS * 256);
 
-    auto finish = [&](int f, f32x4 v) {
+    auto finish = [&](int f, f32x4 v) __attribute__((always_inline)) {
         const int rg = f / MT, mt = f % MT;
         if (a.split_k == 1) {
             store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g);

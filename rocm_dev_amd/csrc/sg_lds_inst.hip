@@ -11,7 +11,8 @@ namespace sg {
 
 template <int XU, int DEPTH, bool NT, int MODE>
 static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
-    if (threads > (unsigned)lds_launch_bound(SG_MT, SG_RG)) return SG_INVALID_CONFIG;
+    if (threads > (unsigned)(MODE == 0 ? lds_launch_bound(SG_MT, SG_RG) : lds_persistent_launch_bound(SG_MT, SG_RG)))
+        return SG_INVALID_CONFIG;
     void (*kernel)(const StreamArgs) = nullptr;
     if constexpr (MODE == 2) kernel = lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
     else if constexpr (MODE == 3) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;

@@ -110,6 +110,9 @@ constexpr int lds_stage_bytes(int RG, int XU) { return (RG * 4 + XU) * 1024; }
 // Eight or more accumulator fragments per wave need more than the 128 VGPRs a 16-wave workgroup
 // leaves each wave; those instantiations accept at most 8 waves per workgroup.
 constexpr int lds_launch_bound(int MT, int RG) { return RG * MT >= 8 ? 512 : 1024; }
+// The persistent kernels recompute their DMA addresses per stage instead of keeping one pointer
+// per instruction, which costs temporaries: four fragments already overflow 128 VGPRs there.
+constexpr int lds_persistent_launch_bound(int MT, int RG) { return RG * MT >= 4 ? 512 : 1024; }
 
 // XU = activation DMA instructions per stage (4 rows each): ceil(min(m, 16*MT) / 4)
 template <int MT, int RG, int XU, int DEPTH, bool NT>
@@ -169,7 +172,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
     const unsigned my_ring_lds = lds_addr(my_ring);
 
-    auto issue = [&](int i) {  // i-th stage of this wave -> slot i % DEPTH
+    auto issue = [&](int i) __attribute__((always_inline)) {  // i-th stage of this wave -> slot i % DEPTH
         const size_t koff = (size_t)(b_begin + wave + i * waves) << 8;
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
 #pragma unroll
@@ -189,7 +192,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto consume = [&](int i) {
+    auto consume = [&](int i) __attribute__((always_inline)) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
         mma_block_256<MT, RG>(slot, slot + RG * 4096, acc);
     };
@@ -230,7 +233,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
 // The reduction scratch is double-buffered by tile parity, which leaves one barrier per tile.
 // No cross-workgroup split-K in this variant.
 template <int MT, int RG, int XU, int DEPTH, bool NT, bool XRES>
-__global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_kernel(const StreamArgs a) {
+__global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_persistent_kernel(const StreamArgs a) {
     // XRES: [X blocks][XU KB] | [wave][DEPTH][RG*4 KB] | red;  else: [wave][DEPTH][(RG*4 + XU) KB] | red[2][FRAGS][wave][64]
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
 
@@ -264,13 +267,13 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
     const unsigned my_ring_lds = lds_addr(my_ring);
     f32x4* red = reinterpret_cast<f32x4*>(ring + x_bytes + (size_t)waves * (DEPTH * STAGE_BYTES));
 
-    auto tile_origin = [&](int j, int& m0, int& n0) {  // j-th tile of this workgroup
+    auto tile_origin = [&](int j, int& m0, int& n0) __attribute__((always_inline)) {  // j-th tile of this workgroup
         const int t = (int)blockIdx.x + j * (int)gridDim.x;
         n0 = (t % a.n_tiles) * (16 * RG);
         m0 = (t / a.n_tiles) * (16 * MT);
     };
 
-    auto issue = [&](int i) {
+    auto issue = [&](int i) __attribute__((always_inline)) {
         const int j = i / per_tile;
         const int kb = wave + (i - j * per_tile) * waves;
         int m0, n0;
@@ -304,7 +307,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
         for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     int left_in_tile = per_tile;  // stages of the current tile not yet consumed
-    auto consume = [&](int i) {
+    auto consume = [&](int i) __attribute__((always_inline)) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
         // activations: in the stage, or in the resident copy at this stage's K block
         const uint8_t* xs = XRES ? ring + (size_t)(wave + (per_tile - left_in_tile) * waves) * (XU * 1024) + rd_off
@@ -314,7 +317,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
 
     const float scale = a.scale ? a.scale[0] : 1.0f;
     // Reduce the waves' partial tiles of the j-th tile in wave order, scale, round, store.
-    auto tile_done = [&](int j) {
+    auto tile_done = [&](int j) __attribute__((always_inline)) {
         int m0, n0;
         tile_origin(j, m0, n0);
         if (waves == 1 && !epilogue_wave) {
@@ -377,7 +380,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
 
     // stage i ends a tile when it is this wave's last K block of that tile
     int tile_j = 0;
-    auto after_consume = [&]() {
+    auto after_consume = [&]() __attribute__((always_inline)) {
         if (--left_in_tile == 0) {
             tile_done(tile_j++);
             left_in_tile = per_tile;
@@ -401,7 +404,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
             __builtin_amdgcn_sched_barrier(0);
             after_consume();
         }
-        auto consume_and_close = [&](int ii) {
+        auto consume_and_close = [&](int ii) __attribute__((always_inline)) {
             consume(ii);
             after_consume();
         };
@@ -426,7 +429,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_persistent_
 // (workgroup b, wave w) walks tiles b*W + w, + total waves, ...; its weight ring runs across
 // tile boundaries.
 template <int MT, int RG, int XU, int DEPTH, bool NT>
-__global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_wavetile_kernel(const StreamArgs a) {
+__global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_wavetile_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // X[blocks][XU KB] | [wave][DEPTH][RG*4 KB]
 
     constexpr int PER_STAGE = RG * 4;
@@ -469,7 +472,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_wavetile_ke
         x_issued += XU;
     }
 
-    auto issue = [&](int i) {
+    auto issue = [&](int i) __attribute__((always_inline)) {
         const int j = i / blocks;
         const int kb = i - j * blocks;
         const int n0 = ((gw + j * total_waves) % a.n_tiles) * (16 * RG);
@@ -494,14 +497,14 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_wavetile_ke
         for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     int kb_cur = 0;  // K block of the stage being consumed
-    auto consume = [&](int i) {
+    auto consume = [&](int i) __attribute__((always_inline)) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
         mma_block_256<MT, RG>(slot, ring + (size_t)kb_cur * (XU * 1024) + rd_off, acc);
     };
 
     const float scale = a.scale ? a.scale[0] : 1.0f;
     int tile_j = 0;
-    auto after_consume = [&]() {
+    auto after_consume = [&]() __attribute__((always_inline)) {
         if (++kb_cur == blocks) {   // the tile is complete: scale, round, store, start the next one
             kb_cur = 0;
             const int n0 = ((gw + tile_j * total_waves) % a.n_tiles) * (16 * RG);
@@ -533,7 +536,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_wavetile_ke
             __builtin_amdgcn_sched_barrier(0);
             after_consume();
         }
-        auto consume_and_close = [&](int ii) {
+        auto consume_and_close = [&](int ii) __attribute__((always_inline)) {
             consume(ii);
             after_consume();
         };

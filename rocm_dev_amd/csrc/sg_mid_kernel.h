@@ -89,7 +89,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         xsrc[i] = a.A + (size_t)row * a.k + ((d_pp ^ ((row_l >> 1) & 7)) << 4);
     }
     const unsigned ring_lds = lds_addr(ring);
-    auto issue = [&](int s) {   // s-th K block of this workgroup -> slot s % DEPTH
+    auto issue = [&](int s) __attribute__((always_inline)) {   // s-th K block of this workgroup -> slot s % DEPTH
         const size_t koff = (size_t)(b_begin + s) << 7;
         const unsigned slot = ring_lds + (unsigned)(s % DEPTH) * STAGE_BYTES;
 #pragma unroll
@@ -112,7 +112,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
 #pragma unroll
         for (int mb = 0; mb < MH; mb++) acc[rg][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto consume = [&](int s) {
+    auto consume = [&](int s) __attribute__((always_inline)) {
         const uint8_t* slot = ring + (size_t)(s % DEPTH) * STAGE_BYTES;
         i32x8 x[MH];
 #pragma unroll
@@ -151,7 +151,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
 
     // ---- epilogue --------------------------------------------------------------------------------
     const float scale = a.scale ? a.scale[0] : 1.0f;
-    auto store_all = [&](auto&& get) {
+    auto store_all = [&](auto&& get) __attribute__((always_inline)) {
 #pragma unroll
         for (int rg = 0; rg < RGW; rg++)
 #pragma unroll

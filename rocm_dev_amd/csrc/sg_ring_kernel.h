@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(1024) ring_gemm_kernel(const RingArgs ra) {
     const int total_blocks = blocks * my_tiles;  // running block count of this workgroup
     const unsigned ring_lds = lds_addr(ring);
 
-    auto tile_origin = [&](int j, int& m0, int& n0) {
+    auto tile_origin = [&](int j, int& m0, int& n0) __attribute__((always_inline)) {
         const int t = (int)blockIdx.x + j * (int)gridDim.x;
         n0 = (t % a.n_tiles) * (16 * BL);
         m0 = (t / a.n_tiles) * (16 * MT);
@@ -114,13 +114,13 @@ __global__ void __launch_bounds__(1024) ring_gemm_kernel(const RingArgs ra) {
         const int n_items = is_a ? total_blocks : total_blocks * BL;   // B items: (block, lane) pairs
         const int per_item = is_a ? XU : 4;                            // DMA instructions per item
 
-        auto flag_of = [&](int item) -> volatile int* {
+        auto flag_of = [&](int item) __attribute__((always_inline)) -> volatile int* {
             const int gb = is_a ? item : item / BL;
             const int slot = gb % Q;
             return is_a ? &queue[2 * BL * slot] : &queue[2 * (BL * slot + (item - gb * BL)) + 1];
         };
-        auto phase_of = [&](int item) { return 2 * ((is_a ? item : item / BL) / Q); };
-        auto issue = [&](int item) {
+        auto phase_of = [&](int item) __attribute__((always_inline)) { return 2 * ((is_a ? item : item / BL) / Q); };
+        auto issue = [&](int item) __attribute__((always_inline)) {
             const int gb = is_a ? item : item / BL;
             const int ln = is_a ? 0 : item - gb * BL;
             const int j = gb / blocks;

@@ -7,6 +7,7 @@ namespace sg {
 
 template <int MT, int RG, int XU2, int DEPTH>
 static int launch_one(const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
+    if (threads > (unsigned)sparse_launch_bound(MT, RG)) return SG_INVALID_CONFIG;
     auto kernel = sparse24_gemm_kernel<MT, RG, XU2, DEPTH>;
     static size_t attr_bytes[16] = {};
     if (lds > 48 * 1024) {

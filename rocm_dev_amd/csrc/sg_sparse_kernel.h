@@ -33,9 +33,13 @@ struct SparseArgs {
     const uint8_t* meta;   // [n][k/8]
 };
 
+// A stage's activation fragments alone take 32*MT registers; two activation blocks or four row
+// tiles per wave do not fit the 128 VGPRs a 16-wave workgroup leaves each wave.
+constexpr int sparse_launch_bound(int MT, int RG) { return (MT == 2 || RG == 4) ? 512 : 1024; }
+
 // XU2 = activation DMA instructions per stage: 2 halves x ceil(rows/4)
 template <int MT, int RG, int XU2, int DEPTH>
-__global__ void __launch_bounds__(1024) sparse24_gemm_kernel(const SparseArgs sa) {
+__global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_kernel(const SparseArgs sa) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
     __shared__ unsigned arrival;
     const StreamArgs& a = sa.g;
@@ -95,7 +99,7 @@ __global__ void __launch_bounds__(1024) sparse24_gemm_kernel(const SparseArgs sa
 
     const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
     const unsigned my_ring_lds = lds_addr(my_ring);
-    auto issue = [&](int i) {
+    auto issue = [&](int i) __attribute__((always_inline)) {
         const size_t kb = (size_t)(b_begin + wave + i * waves);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
 #pragma unroll
@@ -120,7 +124,7 @@ __global__ void __launch_bounds__(1024) sparse24_gemm_kernel(const SparseArgs sa
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto consume = [&](int i) {
+    auto consume = [&](int i) __attribute__((always_inline)) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES;
         i32x4 x[MT][8];
 #pragma unroll
