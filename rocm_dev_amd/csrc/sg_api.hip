@@ -356,7 +356,8 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
     c.mt = m <= 16 ? 1 : 2;
     const int tiles16 = (n + 15) / 16;
     const int blocks = k / 512;
-    c.rg = tiles16 >= 4 * cu_count ? 2 : 1;
+    // above 8 activation rows the activation stage outweighs a 16-row weight stage: share it between two row tiles
+    c.rg = (tiles16 >= 4 * cu_count || (m > 8 && tiles16 >= 2 * cu_count)) ? 2 : 1;
     c.waves = blocks >= 16 ? 2 : 1;
     // many tiles per CU: shallow rings so that several workgroups share a CU
     c.depth = (tiles16 / c.rg >= 2 * cu_count) ? 2 : 4;
