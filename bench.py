@@ -51,6 +51,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs (for counter runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies (known traffic, to scale profiler counters)")
+    ap.add_argument("--mid-batch-counters", action="store_true",
+                    help="only launch the mid-batch GEMMs (M = 64, 128, 256), eagerly, three times each, and exit "
+                         "(for MFMA-utilisation counter runs; prints no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1")
@@ -65,6 +68,21 @@ def main():
     torch.manual_seed(0)
     if lib.sg_init() != 0:
         sys.exit("bench.py: sg_init failed")
+
+    if args.mid_batch_counters:
+        one = torch.ones(1, device="cuda")
+        for (n, k) in ((10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)):
+            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(2)]
+            for m in (64, 128, 256):
+                a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+                d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+                for i in range(3):
+                    rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % 2].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, None)
+                    if rc != 0:
+                        raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
+                torch.cuda.synchronize()
+            del wb
+        return
 
     def quantize(x):
         """Per-tensor scale absmax/448 and OCP E4M3 codes (round to nearest even)."""

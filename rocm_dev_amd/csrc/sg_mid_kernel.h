@@ -11,7 +11,7 @@
 // B/clk/CU) under the MFMA rate.  The MFMA is gfx950's v_mfma_scale_f32_16x16x128_f8f6f4
 // with unit block scales: 128 bytes of K per instruction, i.e. one instruction per stage and
 // fragment pair.  Lane (r = l%16, g = l/16) supplies 32 bytes of row r; which 32 bytes is
-// free as long as both operands agree, so both take 16-byte pieces 2g and 2g+1 of the block.
+// free as long as both operands agree, so both take 16-byte pieces g and g+4 of the block.
 //
 // LDS stage layout: row-major, 128 bytes per row, filled by direct-to-LDS loads of 8 rows x
 // 128 contiguous bytes per instruction.  The 16-byte pieces of a row are XOR-swizzled with
@@ -98,11 +98,13 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         for (int i = 0; i < X_INSTR; i++) dma_1kb(xsrc[i] + koff, slot + BN * 128 + (WAVES * i + wave) * 1024);
     };
 
-    // ---- LDS read offsets: lane (r, g) reads pieces 2g and 2g+1 of row r of a 16-row fragment --
+    // ---- LDS read offsets: lane (r, g) reads pieces g and g+4 of row r of a 16-row fragment ------
     const int r = lane & 15, g = lane >> 4;
-    const int piece0 = ((2 * g) ^ ((r >> 1) & 7)) << 4;
+    // pieces g and g + 4, not 2g and 2g + 1: with the row swizzle above the first choice is free of bank
+    // conflicts at the LDS's full 256 B/clk, the second runs every ds_read_b128 at half rate (measured)
+    const int piece0 = (g ^ ((r >> 1) & 7)) << 4;
     const int rd0 = r * 128 + piece0;
-    const int rd1 = r * 128 + (piece0 ^ 16);
+    const int rd1 = r * 128 + (piece0 ^ 64);
     const int w_base = (wn * RGW * 16) * 128;                   // this wave's weight rows
     const int x_base = BN * 128 + (wm * MH * 16) * 128;         // this wave's activation rows
 
