@@ -97,6 +97,17 @@ int sg_skinny_gemm_fastpath(const uint8_t* A, const uint8_t* B, void* D_bf16, co
 int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
                         int m, int n, int k, int b_stride, void* stream);
 
+/* The same GEMM with per-row and per-column scale factors in the epilogue:
+ *     D[i][j] = bf16( ((sum_k A[i][k]*B[j][k]) * scale) * row_scales[i] * col_scales[j] )
+ * with three separately rounded fp32 products in that order.  No counterpart in the reference (its
+ * epilogue applies the one scalar, skinny_gemm/consumers/mfma_16x16x32_consumer.cu:111-118); this is
+ * the step on either side of the GEMM in a decode layer: activations quantised per row with
+ * sg_fp8_encode_rows (its `scales` output is row_scales), weights quantised per output channel.
+ * scale_tensor, row_scales ([m] floats) and col_scales ([n] floats) may each be NULL (factor 1). */
+int sg_skinny_gemm_rowcol(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                          const float* row_scales, const float* col_scales, int m, int n, int k, int b_stride,
+                          void* stream);
+
 /* Library-native tuning record for sg_skinny_gemm_tuned - no counterpart in the reference,
  * whose tunables are compile-time #defines rewritten by its grid-search script
  * (grid.py:106-116); this is the run-time equivalent a tuning driver sweeps. */

@@ -45,6 +45,7 @@ def _load():
         "orc_quantize_tensor": (f32, [vp, vp, sz]),
         "orc_gemm_ref": (None, [vp, vp, vp, f32, i32, i32, i32, i32]),
         "orc_gemm_omp": (None, [vp, vp, vp, f32, i32, i32, i32, i32]),
+        "orc_gemm_rowcol": (None, [vp, vp, vp, f32, vp, vp, i32, i32, i32, i32]),
         "orc_gemm_f32": (None, [vp, vp, vp, f32, i32, i32, i32, i32]),
         "orc_gemm_f64": (None, [vp, vp, vp, dbl, i32, i32, i32, i32]),
         "orc_num_threads": (i32, []),
@@ -176,6 +177,22 @@ def gemm_ref(A, B, scale):
 def gemm_omp(A, B, scale):
     """Same sums on all cores; bf16 bits out."""
     return _gemm(_lib.orc_gemm_omp, A, B, scale, np.uint16)
+
+
+def gemm_rowcol(A, B, scale=1.0, row_scale=None, col_scale=None):
+    """bf16 bits of ((sum * scale) * row_scale[i]) * col_scale[j]; either vector may be None."""
+    A = _c(A, np.uint8)
+    B = _c(B, np.uint8)
+    m, k = A.shape
+    n = B.shape[0]
+    rs = None if row_scale is None else _c(row_scale, np.float32)
+    cs = None if col_scale is None else _c(col_scale, np.float32)
+    assert rs is None or rs.shape == (m,)
+    assert cs is None or cs.shape == (n,)
+    D = np.empty((m, n), np.uint16)
+    _lib.orc_gemm_rowcol(_p(A), _p(B), _p(D), float(scale), None if rs is None else _p(rs), None if cs is None else _p(cs),
+                         m, n, k, B.shape[1])
+    return D
 
 
 def gemm_f32(A, B, scale=1.0):

@@ -191,6 +191,24 @@ void orc_gemm_omp(const uint8_t* A, const uint8_t* B, uint16_t* D, float scale,
     free(tmp);
 }
 
+/* Per-row x per-column scaled epilogue (no reference counterpart; it generalises the reference's
+ * "scale once after the K sum, cast last", projects/skinny_gemm/test.cu:32-37): the fp32 sum is
+ * multiplied by scale, then by row_scale[i], then by col_scale[j] - three separately rounded fp32
+ * products in that order, absent factors skipped - and rounded to bf16 once. */
+void orc_gemm_rowcol(const uint8_t* A, const uint8_t* B, uint16_t* D, float scale, const float* row_scale,
+                     const float* col_scale, int m, int n, int k, int b_stride) {
+    float* tmp = (float*)malloc((size_t)m * n * sizeof(float));
+    orc_gemm_f32(A, B, tmp, 1.0f, m, n, k, b_stride);
+    for (int i = 0; i < m; i++)
+        for (int j = 0; j < n; j++) {
+            float v = tmp[(size_t)i * n + j] * scale;
+            if (row_scale) v = v * row_scale[i];
+            if (col_scale) v = v * col_scale[j];
+            D[(size_t)i * n + j] = orc_bf16_from_f32(v);
+        }
+    free(tmp);
+}
+
 void orc_gemm_f64(const uint8_t* A, const uint8_t* B, double* D, double scale,
                   int m, int n, int k, int b_stride) {
     float lut[256];

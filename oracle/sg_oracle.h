@@ -65,6 +65,9 @@ void orc_gemm_omp(const uint8_t* A, const uint8_t* B, uint16_t* D, float scale,
 /* fp32 output of the same sum, scale applied (pass 1.0f for the async_gemm flavour) */
 void orc_gemm_f32(const uint8_t* A, const uint8_t* B, float* D, float scale,
                   int m, int n, int k, int b_stride);
+/* bf16( ((sum * scale) * row_scale[i]) * col_scale[j] ), each product rounded to fp32; either array may be NULL */
+void orc_gemm_rowcol(const uint8_t* A, const uint8_t* B, uint16_t* D, float scale, const float* row_scale,
+                     const float* col_scale, int m, int n, int k, int b_stride);
 /* fp64 accumulated truth (no output rounding) */
 void orc_gemm_f64(const uint8_t* A, const uint8_t* B, double* D, double scale,
                   int m, int n, int k, int b_stride);

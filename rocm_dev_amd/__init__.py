@@ -17,6 +17,7 @@ from .api import (  # noqa: F401
     SgTuning,
     skinny_gemm_fastpath,
     skinny_gemm_pick,
+    skinny_gemm_rowcol,
     skinny_gemm_tuned,
     strerror,
     tiled_sum_reduce,

@@ -23,6 +23,7 @@ SIGNATURES = {
     "sg_skinny_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm_fastpath": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "sg_skinny_gemm_auto": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "sg_skinny_gemm_rowcol": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm_tuned": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sg_skinny_gemm_pick": (_i, [_i, _i, _i, C.POINTER(_i * 8)]),
     "sg_async_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i]),

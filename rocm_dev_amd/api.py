@@ -99,6 +99,23 @@ class SgTuning(C.Structure):
 ENGINE_AUTO, ENGINE_DIRECT, ENGINE_LDS = 0, 1, 2
 
 
+def skinny_gemm_rowcol(A, B, D, scale_tensor=None, row_scales=None, col_scales=None, check=False):
+    """D = bf16(((A @ B^T) * scale) * row_scales[:, None] * col_scales[None, :]); any factor may be None."""
+    m, k = A.shape
+    n = B.shape[0]
+    if row_scales is not None and tuple(row_scales.shape) != (m,):
+        raise ValueError("row_scales must have shape (m,)")
+    if col_scales is not None and tuple(col_scales.shape) != (n,):
+        raise ValueError("col_scales must have shape (n,)")
+    with torch.cuda.device(A.device):
+        rc = lib.sg_skinny_gemm_rowcol(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
+                                       None if scale_tensor is None else _dev(scale_tensor, torch.float32),
+                                       None if row_scales is None else _dev(row_scales, torch.float32),
+                                       None if col_scales is None else _dev(col_scales, torch.float32),
+                                       m, n, k, B.stride(0), _stream())
+    return _done(rc, check)
+
+
 def skinny_gemm_tuned(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k=1, waves=4, row_tiles=1, m_blocks=None,
                       depth=2, k_chunks=4, non_temporal=1, persistent_wgs_per_cu=0, wave_tiles=0, check=False):
     """The library-native tuning entry (no reference counterpart): pick the engine and its shape."""

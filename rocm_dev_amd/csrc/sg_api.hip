@@ -624,6 +624,24 @@ int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D, const float
     return launch_config(c, a, static_cast<hipStream_t>(stream));
 }
 
+int sg_skinny_gemm_rowcol(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, const float* row_scales,
+                          const float* col_scales, int m, int n, int k, int b_stride, void* stream) {
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 16 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (int rc = check_pointers(A, B, D, m, n, k, b_stride)) return rc;
+    if ((reinterpret_cast<uintptr_t>(row_scales) | reinterpret_cast<uintptr_t>(col_scales)) & 3u) return SG_BAD_ALIGNMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    const Config c = (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, dev->cu_count) : pick_config(m, n, k, dev->cu_count);
+    StreamArgs a{};
+    a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;   // nullptr = 1.0f
+    a.row_scale = row_scales;
+    a.col_scale = col_scales;
+    a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
+    a.out_f32 = 0;
+    return launch_config(c, a, static_cast<hipStream_t>(stream));
+}
+
 int sg_skinny_gemm_fastpath(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n,
                             int k) {
     return sg_skinny_gemm_auto(A, B, D, scale_tensor, m, n, k, k, nullptr);

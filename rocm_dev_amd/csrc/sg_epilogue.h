@@ -23,6 +23,8 @@ struct StreamArgs {
     const uint8_t* B;
     void* D;                // bf16 or fp32, [m, n]
     const float* scale;     // device scalar, or nullptr for 1.0f
+    const float* row_scale; // [m] per-activation-row factors, or nullptr
+    const float* col_scale; // [n] per-weight-row (output column) factors, or nullptr
     float* ws;              // split-K partials (fp32)
     unsigned* counters;     // one arrival counter per output tile, zero between launches
     int m, n, k, b_stride;
@@ -39,7 +41,14 @@ __device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, flo
     // with the 16x16x128 instruction - and the operand rows supplied by the masked lanes are then garbage.
     asm volatile("" : "+v"(v));
     if (m_idx >= a.m) return;
+    // scale, then the row factor, then the column factors: three separately rounded fp32 products
     v *= scale;
+    if (a.row_scale) v *= a.row_scale[m_idx];
+    if (a.col_scale) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (n_idx + e < a.n) v[e] *= a.col_scale[n_idx + e];
+    }
     const size_t off = (size_t)m_idx * a.n + n_idx;
     if (a.out_f32) {
         float* d = reinterpret_cast<float*>(a.D) + off;

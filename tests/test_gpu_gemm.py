@@ -253,6 +253,59 @@ def test_producer_consumer_ring(sg, oracle, cfg, shape):
         assert np.array_equal(bits(D2), got)
 
 
+@pytest.mark.parametrize("shape", [(8, 4096, 4096), (5, 130, 512), (32, 6144, 1024), (16, 28672, 1024), (64, 512, 1024),
+                                   (200, 258, 2048), (1, 64, 48), (256, 1024, 512)])
+@pytest.mark.parametrize("which", ["both", "rows", "cols", "none"])
+def test_row_and_column_scaled_epilogue(sg, oracle, shape, which):
+    """sg_skinny_gemm_rowcol: scalar, per-activation-row and per-output-column factors in the epilogue."""
+    m, n, k = shape
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=31)
+    rng = np.random.default_rng(m + n + k)
+    rs = rng.uniform(0.25, 4.0, m).astype(np.float32) if which in ("both", "rows") else None
+    cs = rng.uniform(0.25, 4.0, n).astype(np.float32) if which in ("both", "cols") else None
+    ref = oracle.gemm_rowcol(a8, b8, scale, rs, cs)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    R = None if rs is None else torch.from_numpy(rs).cuda()
+    Cs = None if cs is None else torch.from_numpy(cs).cuda()
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_rowcol(A, B, D, S, R, Cs) == 0
+    torch.cuda.synchronize()
+    got = bits(D)
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
+    if which == "none":
+        D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        assert sg.skinny_gemm_fastpath(A, B, D2, S) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(D2), got)
+
+
+def test_encode_rows_feeds_rowcol_gemm(sg, oracle):
+    """The decode-layer sequence: bf16 activations -> per-row E4M3 (sg_fp8_encode_rows) -> GEMM with the
+    row scales that the encoder produced and per-output-channel weight scales."""
+    m, n, k = 8, 1024, 2048
+    x = oracle.normal_f32((m, k), 5, 1)
+    xb = torch.from_numpy(x).bfloat16()
+    w = oracle.normal_f32((n, k), 6, 1)
+    wmax = np.abs(w).max(axis=1)
+    cs = (wmax / 448.0).astype(np.float32)
+    w8 = torch.from_numpy(w / cs[:, None]).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    X = xb.cuda()
+    Q = torch.empty((m, k), dtype=torch.uint8, device="cuda")
+    RS = torch.empty((m,), dtype=torch.float32, device="cuda")
+    assert sg.fp8_encode_rows(X, Q, RS) == 0
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_rowcol(Q, dev(w8), D, None, RS, torch.from_numpy(cs).cuda()) == 0
+    torch.cuda.synchronize()
+    q_ref, s_ref = oracle.fp8_encode_rows(xb.view(torch.int16).numpy().view(np.uint16))
+    assert np.array_equal(Q.cpu().numpy(), q_ref) and np.array_equal(RS.cpu().numpy(), s_ref)
+    ref = oracle.gemm_rowcol(q_ref, w8, 1.0, s_ref, cs)
+    assert oracle.max_rel_err_bf16(bits(D), ref) <= gemm_tol(k)
+    # and the result approximates the unquantised product
+    exact = xb.float().numpy().astype(np.float64) @ w.astype(np.float64).T
+    got = oracle.bf16_to_f32(bits(D)).astype(np.float64)
+    assert np.abs(got - exact).max() <= 0.08 * np.abs(exact).max()
+
+
 MID_CONFIGS = [
     # row_tiles (RGW), m_blocks (MH), depth, split_k, waves
     (2, 2, 2, 1, 4),

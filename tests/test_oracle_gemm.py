@@ -62,6 +62,37 @@ def test_sequential_order_is_what_is_restated(oracle):
     assert np.array_equal(oracle.gemm_ref(A, B, scale), _bf16(want))
 
 
+def test_rowcol_epilogue_pinned(oracle):
+    """Per-row x per-column scaled epilogue: numpy float32 products in the stated order (bit-exact),
+    reductions to the scalar case, and an asymmetric check that catches swapped row/column vectors."""
+    rng = np.random.default_rng(17)
+    m, n, k = 5, 12, 96
+    A, B = _rand_codes(rng, (m, k)), _rand_codes(rng, (n, k))
+    scale = np.float32(3.1e-3)
+    rs = rng.uniform(0.25, 4.0, m).astype(np.float32)
+    cs = rng.uniform(0.25, 4.0, n).astype(np.float32)
+    acc = oracle.gemm_f32(A, B, 1.0)                       # the fp32 sums themselves (pinned above)
+    want = ((acc * scale).astype(np.float32) * rs[:, None]).astype(np.float32)
+    want = (want * cs[None, :]).astype(np.float32)
+    assert np.array_equal(oracle.gemm_rowcol(A, B, scale, rs, cs), _bf16(want))
+    # absent factors are skipped, and all-ones vectors change nothing
+    assert np.array_equal(oracle.gemm_rowcol(A, B, scale), oracle.gemm_omp(A, B, scale))
+    assert np.array_equal(oracle.gemm_rowcol(A, B, scale, np.ones(m, np.float32), np.ones(n, np.float32)),
+                          oracle.gemm_omp(A, B, scale))
+    only_r = (acc * scale).astype(np.float32) * rs[:, None]
+    assert np.array_equal(oracle.gemm_rowcol(A, B, scale, rs, None), _bf16(only_r.astype(np.float32)))
+    # powers of two commute with every rounding: scaling row 2 by 8 and column 3 by 1/4 is exact
+    r2 = np.ones(m, np.float32); r2[2] = 8.0
+    c2 = np.ones(n, np.float32); c2[3] = 0.25
+    base = oracle.bf16_to_f32(oracle.gemm_omp(A, B, scale))
+    got = oracle.bf16_to_f32(oracle.gemm_rowcol(A, B, scale, r2, c2))
+    expect = base.copy(); expect[2, :] *= 8.0; expect[:, 3] *= 0.25
+    assert np.array_equal(got, expect)
+    # against fp64 truth
+    truth = (_dec(A) @ _dec(B).T) * float(scale) * rs[:, None].astype(np.float64) * cs[None, :].astype(np.float64)
+    assert np.allclose(oracle.bf16_to_f32(oracle.gemm_rowcol(A, B, scale, rs, cs)), truth, rtol=2 ** -7, atol=1e-30)
+
+
 def test_invariants(oracle):
     rng = np.random.default_rng(11)
     m, n, k = 8, 32, 64
