@@ -161,6 +161,13 @@ int sg_sparse24_gemm(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_m
 int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D_bf16,
                            const float* scale_tensor, int m, int n, int k, const SgTuning* tuning, void* stream);
 
+/* Producer of that format: prunes a dense E4M3 matrix B [n][k] (row stride b_stride) to 2:4 and
+ * compresses it.  Per group of four consecutive k the two codes of largest magnitude are kept
+ * (ties keep the lower position; an already-2:4 input is compressed unchanged, zeros padding with the
+ * lowest free positions).  No counterpart in the reference.  k % 16 == 0; B 16-byte aligned with
+ * b_stride % 16 == 0, B_vals 8-byte, B_meta 2-byte aligned. */
+int sg_sparse24_compress(const uint8_t* B, uint8_t* B_vals, uint8_t* B_meta, int n, int k, int b_stride, void* stream);
+
 /* Replaces  void tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m,
  * int n)  (tiled_sum_reduce/src.cu:52-73):  D[m,n] = sum_b (A[b,m,n] + B[b,m,n]), summed
  * in batch order per element.  Any m, n (the reference needs m % 8 == 0, n % 64 == 0). */

@@ -45,6 +45,7 @@ def _load():
         "orc_quantize_tensor": (f32, [vp, vp, sz]),
         "orc_gemm_ref": (None, [vp, vp, vp, f32, i32, i32, i32, i32]),
         "orc_gemm_omp": (None, [vp, vp, vp, f32, i32, i32, i32, i32]),
+        "orc_prune24_e4m3": (None, [vp, i32, i32]),
         "orc_gemm_rowcol": (None, [vp, vp, vp, f32, vp, vp, i32, i32, i32, i32]),
         "orc_gemm_f32": (None, [vp, vp, vp, f32, i32, i32, i32, i32]),
         "orc_gemm_f64": (None, [vp, vp, vp, dbl, i32, i32, i32, i32]),
@@ -214,6 +215,15 @@ def prune24(B):
     assert k % 4 == 0
     _lib.orc_prune24_f32(_p(B), n, k)
     return B
+
+
+def prune24_e4m3(B8):
+    """2:4 prune on E4M3 codes: keep the two largest magnitudes (code & 0x7f) per group of four, ties -> lower index."""
+    B8 = np.array(B8, dtype=np.uint8, order="C", copy=True)
+    n, k = B8.shape
+    assert k % 4 == 0
+    _lib.orc_prune24_e4m3(_p(B8), n, k)
+    return B8
 
 
 def compress24(B8):

@@ -248,6 +248,19 @@ void orc_prune24_f32(float* B, int n, int k) {
     }
 }
 
+/* The same rule on E4M3 codes: |x| is ordered by the low seven bits of the code (sign dropped;
+ * the NaN code 0x7f sorts last and would be kept), dropped positions become +0. */
+void orc_prune24_e4m3(uint8_t* B, int n, int k) {
+#pragma omp parallel for schedule(static)
+    for (long long g = 0; g < (long long)n * (k / 4); g++) {
+        uint8_t* p = B + 4 * g;
+        int i0 = -1, i1 = -1;
+        for (int i = 0; i < 4; i++) if (i0 < 0 || (p[i] & 0x7f) > (p[i0] & 0x7f)) i0 = i;
+        for (int i = 0; i < 4; i++) if (i != i0 && (i1 < 0 || (p[i] & 0x7f) > (p[i1] & 0x7f))) i1 = i;
+        for (int i = 0; i < 4; i++) if (i != i0 && i != i1) p[i] = 0;
+    }
+}
+
 int orc_compress24(const uint8_t* B, uint8_t* vals, uint8_t* meta, int n, int k) {
     size_t groups = (size_t)n * (k / 4);
     int bad = 0;

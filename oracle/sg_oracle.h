@@ -76,6 +76,8 @@ int  orc_num_threads(void);
 /* ---- 2:4 structured sparsity (weights N x K, groups of 4 along K) ------- */
 /* keep the 2 largest |x| of each group, ties -> lower index; zeros the rest in place */
 void orc_prune24_f32(float* B, int n, int k);
+/* the same rule applied to E4M3 codes (magnitude = code & 0x7f); dropped positions become 0x00 */
+void orc_prune24_e4m3(uint8_t* B, int n, int k);
 /* dense E4M3 N x K (already 2:4) -> values N x K/2 + metadata N x K/8.
  * One nibble per group: low 2 bits = index of first kept value, high 2 bits =
  * index of the second (first < second); two groups per byte, lower group in the

@@ -13,6 +13,7 @@ from .api import (  # noqa: F401
     fp8_encode_rows,
     fp8_reduce_rows,
     skinny_gemm,
+    sparse24_compress,
     sparse24_gemm,
     SgTuning,
     skinny_gemm_fastpath,

@@ -179,6 +179,16 @@ def sparse24_gemm(A, B_vals, B_meta, D, scale_tensor, tuning=None, check=False):
     return _done(rc, check)
 
 
+def sparse24_compress(B, B_vals, B_meta, check=False):
+    """Prune dense E4M3 weights B [n, k] to 2:4 (two largest magnitudes per group of four) and compress them
+    into B_vals [n, k/2] and B_meta [n, k/8] (format of include/sgemm.h)."""
+    n, k = B.shape
+    with torch.cuda.device(B.device):
+        rc = lib.sg_sparse24_compress(_dev(B, *_FP8), _dev(B_vals, *_FP8), _dev(B_meta, torch.uint8), n, k, B.stride(0),
+                                      _stream())
+    return _done(rc, check)
+
+
 def async_gemm(A, B, D, check=False):
     """D = A @ B^T without a scale on the default stream; D is float32 or bfloat16."""
     m, k = A.shape

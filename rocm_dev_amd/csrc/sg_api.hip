@@ -17,6 +17,7 @@ int launch_fp8_decode_rows(const uint8_t* Q, const float* scales, void* Y, int r
 int launch_fp8_reduce_rows(const uint8_t* Q, const float* scales, void* Y, int nbuf, size_t q_buf_stride, int rows,
                            int cols, hipStream_t stream);
 int launch_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n, hipStream_t stream);
+int launch_sparse24_compress(const uint8_t* B, uint8_t* vals, uint8_t* meta, int n, int k, int b_stride, hipStream_t stream);
 
 // ---- per-device state -------------------------------------------------------------------
 constexpr int kMaxDevices = 16;
@@ -698,6 +699,17 @@ int sg_sparse24_gemm(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_m
     a.m = m; a.n = n; a.k = k; a.b_stride = k / 2;
     a.out_f32 = 0;
     return launch_sparse_engine(c, a, B_meta, static_cast<hipStream_t>(stream));
+}
+
+int sg_sparse24_compress(const uint8_t* B, uint8_t* B_vals, uint8_t* B_meta, int n, int k, int b_stride, void* stream) {
+    if (!B || !B_vals || !B_meta || n <= 0 || k <= 0 || b_stride < k) return SG_BAD_ARGUMENT;
+    if (k % 16 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if ((reinterpret_cast<uintptr_t>(B) & 15u) || (b_stride & 15) || (reinterpret_cast<uintptr_t>(B_vals) & 7u) ||
+        (reinterpret_cast<uintptr_t>(B_meta) & 1u))
+        return SG_BAD_ALIGNMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    return launch_sparse24_compress(B, B_vals, B_meta, n, k, b_stride, static_cast<hipStream_t>(stream));
 }
 
 int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D,

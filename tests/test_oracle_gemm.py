@@ -181,6 +181,34 @@ def test_prune24_independent(oracle):
     assert ((got.reshape(-1, 4) != 0).sum(1) <= 2).all()
 
 
+def test_prune24_on_codes_independent(oracle):
+    """Prune on E4M3 codes: stable argsort of the magnitude bits; agrees with the float prune wherever the
+    decoded magnitudes of a group are pairwise different."""
+    rng = np.random.default_rng(19)
+    B8 = _rand_codes(rng, (32, 128))
+    B8[0, :4] = [0x38, 0xB8, 0x38, 0x30]      # +1, -1, +1, +0.5: tie keeps positions 0 and 1
+    B8[1, :4] = [0x00, 0x80, 0x00, 0x00]      # zeros of both signs: keeps 0 and 1, stored as 0x00 / 0x80
+    B8[2, :4] = [0x40, 0x44, 0xC4, 0x40]      # 2, 3, -3, 2: keeps 1 and 2
+    got = oracle.prune24_e4m3(B8)
+    g = B8.reshape(-1, 4)
+    order = np.argsort(-(g & 0x7F).astype(np.int32), axis=1, kind="stable")[:, :2]
+    want = np.zeros_like(g)
+    rows = np.arange(g.shape[0])[:, None]
+    want[rows, order] = g[rows, order]
+    assert np.array_equal(got, want.reshape(B8.shape))
+    assert list(got[0, :4]) == [0x38, 0xB8, 0, 0] and list(got[2, :4]) == [0, 0x44, 0xC4, 0]
+    # cross-check against the float rule on groups without magnitude ties
+    dec = _dec(B8).astype(np.float32)
+    mags = np.abs(dec).reshape(-1, 4)
+    distinct = np.array([len(set(r)) == 4 for r in mags])
+    fl = oracle.prune24(dec).reshape(-1, 4)
+    assert np.array_equal((fl != 0)[distinct], ((got.reshape(-1, 4) & 0x7F) != 0)[distinct])
+    # a pruned matrix compresses without complaint and round-trips
+    vals, meta = oracle.compress24(got)
+    back = oracle.decompress24(vals, meta)
+    assert np.array_equal(back & 0x7F, got & 0x7F) and np.array_equal(_dec(back), _dec(got))
+
+
 def test_compress24_known_answer_and_roundtrip(oracle):
     B = np.zeros((1, 16), np.uint8)
     B[0, 0:4] = [0x38, 0, 0, 0x40]     # kept idx 0,3 -> nibble 0b1100 = 0xC
