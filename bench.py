@@ -294,7 +294,7 @@ def main():
                 d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
                 one = torch.ones(1, device="cuda")
                 us = graph_time_us(lambda i, st: lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(),
-                                                                         one.data_ptr(), m, n, k, k, st), 2 * copies)
+                                                                         one.data_ptr(), m, n, k, k, st), max(2 * copies, 8))
                 mid.append({"m": m, "n": n, "k": k, "us": round(us, 2), "TBps": round(gemm_bytes(m, n, k) / us / 1e6, 3),
                             "TFLOPs": round(2.0 * m * n * k / us / 1e6, 1), "frac_fp8_peak": round(2.0 * m * n * k / us / 1e6 / 5000.0, 4)})
             del wb
@@ -312,7 +312,7 @@ def main():
                 d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
                 one = torch.ones(1, device="cuda")
                 us = graph_time_us(lambda i, st: lib.sg_sparse24_gemm(a8.data_ptr(), vb[i % copies].data_ptr(), mb[i % copies].data_ptr(),
-                                                                      d.data_ptr(), one.data_ptr(), m, n, k, st), 2 * copies)
+                                                                      d.data_ptr(), one.data_ptr(), m, n, k, st), max(2 * copies, 8))
                 nb = m * k + 0.625 * n * k + 2 * m * n
                 sp.append({"m": m, "n": n, "k": k, "us": round(us, 2), "TBps": round(nb / us / 1e6, 3)})
             del vb, mb

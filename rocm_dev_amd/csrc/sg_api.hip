@@ -361,7 +361,7 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
     c.rg = (tiles16 >= 4 * cu_count || (m > 8 && tiles16 >= 2 * cu_count)) ? 2 : 1;
     c.waves = blocks >= 16 ? 2 : 1;
     // many tiles per CU: shallow rings so that several workgroups share a CU
-    c.depth = (tiles16 / c.rg >= 2 * cu_count) ? 2 : 4;
+    c.depth = (c.rg == 2 || tiles16 / c.rg >= 2 * cu_count) ? 2 : 4;
     const int xu2 = c.mt == 2 ? 16 : ((m + 3) / 4 <= 1 ? 2 : ((m + 3) / 4 <= 2 ? 4 : 8));
     while (c.depth > 2 && ((c.depth - 1) * (c.rg * 5 + xu2) > 63 ||
                            (size_t)c.waves * c.depth * (c.rg * 5 + xu2) * 1024 + 8192 > 159 * 1024))
