@@ -92,7 +92,8 @@ struct Config {
     int engine;   // ENGINE_DIRECT: global -> VGPR -> MFMA;  ENGINE_LDS: global -> LDS ring (DMA) -> MFMA
     int mt;       // 16-row activation blocks per tile (1 or 2)
     int rg;       // 16-row weight tiles per wave
-    int ku;       // direct engine: 64-byte K chunks per stage (the LDS engine's stage is 256 bytes)
+    int ku;       // direct engine: 64-byte K chunks per stage (the LDS engine's stage is 256 bytes);
+                  // mid-batch engine: ring slots of the activations (0 = depth)
     int depth;    // stages in flight per wave
     int waves;    // waves per workgroup, splitting K among themselves
     int split_k;  // workgroups per tile, splitting K among themselves
@@ -265,9 +266,11 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
         a.ws = w->partials;
         a.counters = w->counters;
     }
-    const size_t lds = (size_t)c.depth * (bn + bm) * 128 + (c.split_k > 1 ? 16 : 0);
+    // c.ku: ring slots of the activations (0 or out of range = as many as the weights')
+    const int dx = (c.ku >= 2 && c.ku < c.depth) ? c.ku : c.depth;
+    const size_t lds = ((size_t)c.depth * bn + (size_t)dx * bm) * 128 + (c.split_k > 1 ? 16 : 0);
     if (lds > 160 * 1024) return SG_INVALID_CONFIG;
-    return launch_mid(c.rg, c.mt, c.depth, wn, a, (unsigned)(tiles * c.split_k), lds, stream);
+    return launch_mid(c.rg, c.mt, c.depth, dx, wn, a, (unsigned)(tiles * c.split_k), lds, stream);
 }
 
 // Mid-batch heuristic, fitted to timings of the Llama-3-70B projection shapes at M = 64..256:
@@ -318,11 +321,30 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     c.nt = 1;
     c.persist = 0;
     c.wavetile = 0;
-    c.ku = 2;
     const int bn = 8 * c.rg * c.waves, bm = 32 * c.mt;
-    const int per_wave = (bn + bm) / (8 * c.waves);   // DMA instructions per wave and stage
-    c.depth = co_resident ? 2 : 4;
-    while (c.depth > 2 && ((size_t)c.depth * (bn + bm) * 128 > 159 * 1024 || (c.depth - 2) * per_wave > 63)) c.depth--;
+    const int per_wave_w = bn / (8 * c.waves), per_wave_x = bm / (8 * c.waves);   // DMA instructions per wave and stage
+    // (weight slots, activation slots; 0 = as many): the deepest ring that fits 160 KB.  A shallower
+    // activation ring (activations come from L2, weights from HBM) is what lets the 256 x 256 tile keep
+    // two weight stages in flight.
+    static const int rings[][2] = {{4, 0}, {3, 0}, {3, 2}, {2, 0}};
+    c.depth = 2;
+    c.ku = 0;
+    if (co_resident) {
+        c.depth = 4;
+        c.ku = 2;
+    } else {
+        for (const auto& r : rings) {
+            const int dw = r[0], dx = r[1] ? r[1] : r[0];
+            const int in_flight_x = per_wave_w + (dx - 2) * (per_wave_w + per_wave_x);
+            const int in_flight_w = (dw - 2) * (per_wave_w + per_wave_x);
+            const size_t lds = ((size_t)dw * bn + (size_t)dx * bm) * 128 + (c.split_k > 1 ? 16 : 0);   // + arrival word
+            if (lds > 160 * 1024) continue;
+            if ((in_flight_x < in_flight_w ? in_flight_x : in_flight_w) > 63) continue;
+            c.depth = dw;
+            c.ku = r[1];
+            break;
+        }
+    }
     return c;
 }
 

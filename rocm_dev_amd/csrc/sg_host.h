@@ -38,7 +38,7 @@ int SG_RING_LAUNCHER(1)(int bl, int xu, int nt, const RingArgs& ra, unsigned gri
 int SG_RING_LAUNCHER(2)(int bl, int xu, int nt, const RingArgs& ra, unsigned grid, unsigned threads, size_t lds,
                         hipStream_t stream);
 
-int launch_mid(int rgw, int mh, int depth, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream);
+int launch_mid(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream);
 
 struct SparseArgs;
 int launch_sparse(int mt, int rg, int xu2, int depth, const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds,

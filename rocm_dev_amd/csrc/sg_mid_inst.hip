@@ -5,9 +5,9 @@
 
 namespace sg {
 
-template <int RGW, int MH, int DEPTH, int WN>
+template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH>
 static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
-    auto kernel = mid_gemm_kernel<RGW, MH, DEPTH, WN>;
+    auto kernel = mid_gemm_kernel<RGW, MH, DEPTH, WN, DX>;
     static size_t attr_bytes[16] = {};
     if (lds > 48 * 1024) {
         int dev = 0;
@@ -27,7 +27,7 @@ static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_
 }
 
 #define SG_CASE(RGW_, MH_, DEPTH_)                                                             \
-    if (rgw == RGW_ && mh == MH_ && depth == DEPTH_) {                                         \
+    if (rgw == RGW_ && mh == MH_ && depth == DEPTH_ && dx == DEPTH_) {                         \
         if (wn == 2) {                                                                         \
             if constexpr ((DEPTH_ - 2) * (RGW_ + MH_) <= 63)                                   \
                 return launch_one<RGW_, MH_, DEPTH_, 2>(a, grid, lds, stream);                 \
@@ -37,14 +37,24 @@ static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_
         if (wn == 4) return launch_one<RGW_, MH_, DEPTH_, 4>(a, grid, lds, stream);            \
         return SG_INVALID_CONFIG;                                                              \
     }
+// eight-wave tiles with a shallower activation ring (dx < depth)
+#define SG_CASE_DX(RGW_, MH_, DEPTH_, DX_)                                                     \
+    if (rgw == RGW_ && mh == MH_ && depth == DEPTH_ && dx == DX_ && wn == 4)                   \
+        return launch_one<RGW_, MH_, DEPTH_, 4, DX_>(a, grid, lds, stream);
 
-int launch_mid(int rgw, int mh, int depth, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
+int launch_mid(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
     SG_CASE(2, 2, 2) SG_CASE(2, 2, 3) SG_CASE(2, 2, 4) SG_CASE(2, 2, 6)
     SG_CASE(2, 4, 2) SG_CASE(2, 4, 3) SG_CASE(2, 4, 4) SG_CASE(2, 4, 6)
     SG_CASE(2, 8, 2) SG_CASE(2, 8, 3) SG_CASE(2, 8, 4)
     SG_CASE(4, 2, 2) SG_CASE(4, 2, 3) SG_CASE(4, 2, 4) SG_CASE(4, 2, 6)
     SG_CASE(4, 4, 2) SG_CASE(4, 4, 3) SG_CASE(4, 4, 4)
     SG_CASE(4, 8, 2) SG_CASE(4, 8, 3)
+    SG_CASE_DX(4, 8, 3, 2)                                            // 256 x 256: 96 + 64 KB
+    SG_CASE_DX(4, 4, 4, 2) SG_CASE_DX(4, 4, 4, 3) SG_CASE_DX(4, 4, 3, 2)   // 256 x 128
+    SG_CASE_DX(4, 2, 4, 2) SG_CASE_DX(4, 2, 4, 3)                     // 256 x 64
+    SG_CASE_DX(2, 8, 4, 2) SG_CASE_DX(2, 8, 3, 2) SG_CASE_DX(2, 8, 6, 2)   // 128 x 256
+    SG_CASE_DX(2, 4, 6, 2) SG_CASE_DX(2, 4, 6, 3) SG_CASE_DX(2, 4, 4, 2)   // 128 x 128
+    SG_CASE_DX(2, 2, 6, 2) SG_CASE_DX(2, 2, 6, 3) SG_CASE_DX(2, 2, 4, 2)   // 128 x 64
     return SG_INVALID_CONFIG;
 }
 

@@ -18,9 +18,10 @@
 // (row/2) & 7 - a permutation that keeps every aligned 64-byte run intact for the memory
 // system - so the sixteen lanes of a ds_read_b128 pass land in sixteen different bank groups.
 //
-// Pipeline: DEPTH stages in LDS, DEPTH-1 in flight; per K block each wave waits for its own
-// DMAs of that block (s_waitcnt vmcnt), one workgroup barrier publishes the stage and retires
-// the previous one, the freed slot is refilled, the stage is consumed.
+// Pipeline: the weights have DEPTH ring slots and the activations DX <= DEPTH; per K block each wave
+// waits for its own DMAs of that block (s_waitcnt vmcnt), one workgroup barrier publishes the stage
+// and retires the previous one, the freed slots are refilled (activations first, so that the newest
+// weight stage may stay in flight behind them), the stage is consumed.
 //
 // K is split across workgroups when there are few tiles; partials meet in the fp32 workspace
 // and the last workgroup to arrive sums them in split order (same scheme as the skinny path).
@@ -35,10 +36,13 @@ namespace sg {
 // RGW: 16-row weight fragments per wave (2 or 4)  -> BN = 32*RGW rows per workgroup
 // MH : 16-row activation fragments per wave (2, 4, 8) -> up to 32*MH activation rows per tile
 // WN : waves along N (2 or 4); the workgroup has WN x 2 waves
-template <int RGW, int MH, int DEPTH, int WN>
+// DX : ring slots of the activations (<= DEPTH, the weights' ring slots).  The weights come from HBM,
+//      the activations from L2 with about half the latency; with DX < DEPTH the LDS a shallower
+//      activation ring frees buys the weights one more stage in flight.
+template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH>
 __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) {
-    // [DEPTH][W rows | X rows][128], then (split-K only) 16 bytes for the arrival broadcast; no static
-    // LDS, so that two workgroups of exactly half the CU's LDS can share a CU
+    // [DEPTH][W rows][128] | [DX][X rows][128], then (split-K only) 16 bytes for the arrival broadcast; no
+    // static LDS, so that two workgroups of exactly half the CU's LDS can share a CU
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
 
     constexpr int WAVES = 2 * WN;
@@ -48,8 +52,14 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     constexpr int X_INSTR = BM / 8 / WAVES;   // ... and for the activations
     static_assert(BN % (8 * WAVES) == 0 && BM % (8 * WAVES) == 0, "stage rows must split evenly over the waves' DMA instructions");
     constexpr int PER_STAGE = W_INSTR + X_INSTR;
-    constexpr int STAGE_BYTES = (BN + BM) * 128;
-    static_assert(DEPTH >= 2 && (DEPTH - 2) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
+    constexpr int W_BYTES = BN * 128, X_BYTES = BM * 128;   // one ring slot of each operand
+    constexpr int RING_BYTES = DEPTH * W_BYTES + DX * X_BYTES;
+    static_assert(DX >= 2 && DX <= DEPTH, "activation ring between two slots and the weight ring's depth");
+    // Per iteration the activations of stage s+DX-1 are issued before the weights of stage s+DEPTH-1, so
+    // behind the last instruction of X(s) and W(s) the queue holds at least this many younger ones:
+    constexpr int IN_FLIGHT_X = W_INSTR + (DX - 2) * PER_STAGE, IN_FLIGHT_W = (DEPTH - 2) * PER_STAGE;
+    constexpr int IN_FLIGHT = IN_FLIGHT_X < IN_FLIGHT_W ? IN_FLIGHT_X : IN_FLIGHT_W;
+    static_assert(IN_FLIGHT <= 63, "ring deeper than vmcnt can count");
 
     const int lane = lane_id();
     const int wave = wave_id();
@@ -89,13 +99,25 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         xsrc[i] = a.A + (size_t)row * a.k + ((d_pp ^ ((row_l >> 1) & 7)) << 4);
     }
     const unsigned ring_lds = lds_addr(ring);
-    auto issue = [&](int s) __attribute__((always_inline)) {   // s-th K block of this workgroup -> slot s % DEPTH
-        const size_t koff = (size_t)(b_begin + s) << 7;
-        const unsigned slot = ring_lds + (unsigned)(s % DEPTH) * STAGE_BYTES;
+    // DMA instruction i of a stage's refill: the activation instructions come first, then the weights'
+    auto issue_one = [&](int i, int sx, int sw) __attribute__((always_inline)) {
+        if (i < X_INSTR) {
+            if (sx < n_blk)
+                dma_1kb(xsrc[i] + ((size_t)(b_begin + sx) << 7),
+                        ring_lds + DEPTH * W_BYTES + (unsigned)(sx % DX) * X_BYTES + (WAVES * i + wave) * 1024);
+        } else {
+            if (sw < n_blk)
+                dma_1kb_stream(wsrc[i - X_INSTR] + ((size_t)(b_begin + sw) << 7),
+                               ring_lds + (unsigned)(sw % DEPTH) * W_BYTES + (WAVES * (i - X_INSTR) + wave) * 1024);
+        }
+    };
+    auto issue_x = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < W_INSTR; i++) dma_1kb_stream(wsrc[i] + koff, slot + (WAVES * i + wave) * 1024);
+        for (int i = 0; i < X_INSTR; i++) issue_one(i, s, 0);
+    };
+    auto issue_w = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < X_INSTR; i++) dma_1kb(xsrc[i] + koff, slot + BN * 128 + (WAVES * i + wave) * 1024);
+        for (int i = X_INSTR; i < PER_STAGE; i++) issue_one(i, 0, s);
     };
 
     // ---- LDS read offsets: lane (r, g) reads pieces g and g+4 of row r of a 16-row fragment ------
@@ -105,8 +127,8 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     const int piece0 = (g ^ ((r >> 1) & 7)) << 4;
     const int rd0 = r * 128 + piece0;
     const int rd1 = r * 128 + (piece0 ^ 64);
-    const int w_base = (wn * RGW * 16) * 128;                   // this wave's weight rows
-    const int x_base = BN * 128 + (wm * MH * 16) * 128;         // this wave's activation rows
+    const int w_base = (wn * RGW * 16) * 128;                   // this wave's weight rows inside a weight slot
+    const int x_base = (wm * MH * 16) * 128;                    // this wave's activation rows inside an activation slot
 
     f32x4 acc[RGW][MH];
 #pragma unroll
@@ -114,40 +136,89 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
 #pragma unroll
         for (int mb = 0; mb < MH; mb++) acc[rg][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto consume = [&](int s) __attribute__((always_inline)) {
-        const uint8_t* slot = ring + (size_t)(s % DEPTH) * STAGE_BYTES;
+    // Consumes stage s and, between the MFMA groups, issues the refill of the slots that stage s-1 left
+    // (activations of stage sx, weights of stage sw).  Issued in one burst after the barrier the eight waves'
+    // DMA instructions queue up at the CU's one texture-address unit and every wave stalls at issue, in
+    // order, in front of its MFMAs; spread over the stage they are absorbed while the matrix cores work.
+    auto consume = [&](int s, int sx, int sw) __attribute__((always_inline)) {
+        const uint8_t* wslot = ring + (size_t)(s % DEPTH) * W_BYTES + w_base;
+        const uint8_t* xslot = ring + (size_t)DEPTH * W_BYTES + (size_t)(s % DX) * X_BYTES + x_base;
+        auto read_frag = [&](const uint8_t* p) __attribute__((always_inline)) {
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(p + rd0);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(p + rd1);
+            return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        };
+        // the wave's weight fragments stay in registers for the stage; its activation fragments are
+        // streamed one ahead of the MFMAs that use them, so that only the first reads of a stage are
+        // exposed and the rest of the LDS traffic runs under the matrix cores
+        i32x8 w[RGW];
+#pragma unroll
+        for (int rg = 0; rg < RGW; rg++) w[rg] = read_frag(wslot + rg * 2048);
+        i32x8 x[2];
+        x[0] = read_frag(xslot);
+#pragma unroll
+        for (int mb = 0; mb < MH; mb++) {
+            if (mb + 1 < MH) x[(mb + 1) & 1] = read_frag(xslot + (mb + 1) * 2048);
+#pragma unroll
+            for (int i = mb * PER_STAGE / MH; i < (mb + 1) * PER_STAGE / MH; i++) issue_one(i, sx, sw);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int rg = 0; rg < RGW; rg++)
+                // formats 0/0 = OCP E4M3 for both operands; E8M0 scale byte 127 = 2^0 for both
+                acc[rg][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w[rg], x[mb & 1], acc[rg][mb], 0, 0, 0,
+                                                                               0x7f7f7f7f, 0, 0x7f7f7f7f);
+            // an MFMA has no side effects and its result is not read before the next stage, so the
+            // optimizer would sink the group behind the reads and (conditional) refills that follow, and
+            // hoist every read to the top; naming the accumulators as operands of an asm with a memory
+            // clobber keeps each group, and the reads around it, where they are written
+#pragma unroll
+            for (int rg = 0; rg < RGW; rg++) asm volatile("" : "+v"(acc[rg][mb])::"memory");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // Four-wave workgroups (one wave per SIMD) measure faster the plain way: refill in one burst after the
+    // barrier, all activation fragments read up front, weight fragments one by one.
+    auto consume_burst = [&](int s, int sx, int sw) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < PER_STAGE; i++) issue_one(i, sx, sw);
+        __builtin_amdgcn_sched_barrier(0);
+        const uint8_t* wslot = ring + (size_t)(s % DEPTH) * W_BYTES + w_base;
+        const uint8_t* xslot = ring + (size_t)DEPTH * W_BYTES + (size_t)(s % DX) * X_BYTES + x_base;
         i32x8 x[MH];
 #pragma unroll
         for (int mb = 0; mb < MH; mb++) {
-            const i32x4 lo = *reinterpret_cast<const i32x4*>(slot + x_base + mb * 2048 + rd0);
-            const i32x4 hi = *reinterpret_cast<const i32x4*>(slot + x_base + mb * 2048 + rd1);
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(xslot + mb * 2048 + rd0);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(xslot + mb * 2048 + rd1);
             x[mb] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
         }
 #pragma unroll
         for (int rg = 0; rg < RGW; rg++) {
-            const i32x4 lo = *reinterpret_cast<const i32x4*>(slot + w_base + rg * 2048 + rd0);
-            const i32x4 hi = *reinterpret_cast<const i32x4*>(slot + w_base + rg * 2048 + rd1);
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(wslot + rg * 2048 + rd0);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(wslot + rg * 2048 + rd1);
             const i32x8 w = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
             for (int mb = 0; mb < MH; mb++)
-                // formats 0/0 = OCP E4M3 for both operands; E8M0 scale byte 127 = 2^0 for both
                 acc[rg][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, x[mb], acc[rg][mb], 0, 0, 0, 0x7f7f7f7f,
                                                                                0, 0x7f7f7f7f);
         }
     };
 
     // ---- pipeline ------------------------------------------------------------------------------
-    const int prologue = n_blk < DEPTH - 1 ? n_blk : DEPTH - 1;
-    for (int s = 0; s < prologue; s++) issue(s);
+    for (int i = 0; i < DEPTH - 1; i++) {
+        if (i < DX - 1 && i < n_blk) issue_x(i);
+        if (i < n_blk) issue_w(i);
+    }
     for (int s = 0; s < n_blk; s++) {
-        // stages s .. min(s + DEPTH - 2, n_blk - 1) are in flight; wait for this wave's part of stage s
-        const int younger = (n_blk - 1 - s) < (DEPTH - 2) ? (n_blk - 1 - s) : (DEPTH - 2);
-        if (younger == DEPTH - 2) wait_vmcnt<(DEPTH - 2) * PER_STAGE>();
-        else wait_vmcnt<0>();   // tail of the K range: fewer stages behind this one
+        // wait for this wave's part of stage s; everything issued after it may stay in flight.  Near the
+        // end of the K range fewer stages follow, and the count is no longer known at compile time.
+        if (s + DEPTH - 2 < n_blk) wait_vmcnt<IN_FLIGHT>();
+        else wait_vmcnt<0>();
         __syncthreads();        // stage s is complete for every wave; stage s-1 has been consumed by every wave
-        if (s + DEPTH - 1 < n_blk) issue(s + DEPTH - 1);   // refill the slot of stage s-1
         __builtin_amdgcn_sched_barrier(0);
-        consume(s);
+        // refills the slots of X(s-1) and W(s-1) on the way
+        if constexpr (WN == 2) consume_burst(s, s + DX - 1, s + DEPTH - 1);
+        else consume(s, s + DX - 1, s + DEPTH - 1);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
 
@@ -182,7 +253,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    volatile unsigned* arrival = reinterpret_cast<volatile unsigned*>(ring + (size_t)DEPTH * STAGE_BYTES);
+    volatile unsigned* arrival = reinterpret_cast<volatile unsigned*>(ring + (size_t)RING_BYTES);
     if (threadIdx.x == 0)
         *arrival = __hip_atomic_fetch_add(&a.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();

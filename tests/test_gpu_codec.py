@@ -46,7 +46,7 @@ def test_encode_bit_exact(sg, oracle, rows, cols):
 
 
 def test_encode_decode_reduce_config3_slice(sg, oracle):
-    """BASELINE config 3 recipe on a 512-row slice: 8 seeded buffers, outliers, encode, reduce."""
+    """benchmark configuration 3 recipe on a 512-row slice: 8 seeded buffers, outliers, encode, reduce."""
     nbuf, rows, cols = 8, 512, 8192
     Q = torch.empty((nbuf, rows, cols), dtype=torch.uint8, device="cuda")
     S = torch.empty((nbuf, rows), dtype=torch.float32, device="cuda")
@@ -89,7 +89,7 @@ def test_reduce_other_counts(sg, oracle, nbuf):
 
 
 def test_full_size_properties(sg, oracle):
-    """8192 x 8192 (BASELINE config 3 size): properties that need no full-size oracle pass,
+    """8192 x 8192 (benchmark configuration 3 size): properties that need no full-size oracle pass,
     plus the oracle on the first and last 64 rows."""
     rows = cols = 8192
     g = torch.Generator(device="cuda").manual_seed(0)

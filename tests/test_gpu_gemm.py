@@ -30,7 +30,7 @@ def _run_fast(sg, a8, b8, scale):
 
 
 def test_config1_fastpath(sg, oracle):
-    """BASELINE config 1: 8 x 4096 x 4096, N(0,1) seed 0, per-tensor scales."""
+    """benchmark configuration 1: 8 x 4096 x 4096, N(0,1) seed 0, per-tensor scales."""
     a8, b8, scale = oracle.make_gemm_operands(8, 4096, 4096, seed=0)
     ref = oracle.gemm_omp(a8, b8, scale)
     got = _run_fast(sg, a8, b8, scale)
@@ -321,6 +321,12 @@ MID_CONFIGS = [
     (2, 8, 3, 4, 8),
     (4, 8, 2, 1, 8),
     (4, 2, 6, 2, 8),
+    # ... with a shallower activation ring (sixth entry)
+    (4, 8, 3, 1, 8, 2),
+    (4, 4, 4, 2, 8, 2),
+    (2, 8, 4, 1, 8, 2),
+    (2, 4, 6, 1, 8, 3),
+    (2, 2, 4, 4, 8, 2),
 ]
 
 
@@ -329,13 +335,14 @@ MID_CONFIGS = [
                                    (300, 128, 1536), (33, 64, 128)])
 def test_mid_batch_engine(sg, oracle, cfg, shape):
     """32 < m: weights streamed once, 2 x 2 or 4 x 2 waves per tile, 16x16x128 scaled MFMA with unit scales."""
-    rgw, mh, depth, split_k, waves = cfg
+    rgw, mh, depth, split_k, waves = cfg[:5]
+    dx = cfg[5] if len(cfg) > 5 else 0
     m, n, k = shape
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=11)
     ref = oracle.gemm_omp(a8, b8, scale)
     A, B, S = dev(a8), dev(b8), scale_tensor(scale)
     D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
-    kw = dict(engine=4, split_k=split_k, waves=waves, row_tiles=rgw, m_blocks=mh, depth=depth)
+    kw = dict(engine=4, split_k=split_k, waves=waves, row_tiles=rgw, m_blocks=mh, depth=depth, k_chunks=dx)
     rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
     torch.cuda.synchronize()
     if rc == 6:
@@ -352,7 +359,7 @@ def test_mid_batch_engine(sg, oracle, cfg, shape):
 @pytest.mark.parametrize("m,n,k", [(64, 10240, 8192), (128, 10240, 8192), (128, 8192, 8192), (256, 8192, 8192),
                                    (128, 57344, 8192), (256, 57344, 8192), (64, 8192, 28672), (256, 8192, 28672)])
 def test_mid_batch_config4_shapes(sg, oracle, m, n, k):
-    """BASELINE config 4 shapes at full size through the fastpath.  The oracle checks two
+    """benchmark configuration 4 shapes at full size through the fastpath.  The oracle checks two
     512-row slices of the weight matrix (tiles are independent along n); the rest is covered
     by linearity: doubling the scale doubles every output exactly."""
     a = oracle.normal_f32((m, k), 0, 1)
@@ -474,7 +481,7 @@ def test_async_gemm(sg, oracle):
 @pytest.mark.parametrize("n,k", [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)])
 @pytest.mark.parametrize("m", [1, 8, 32])
 def test_decode_sweep_shapes(sg, oracle, m, n, k):
-    """BASELINE config 2 shapes at full size (the oracle on all cores takes about a second each)."""
+    """benchmark configuration 2 shapes at full size (the oracle on all cores takes about a second each)."""
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=0)
     ref = oracle.gemm_omp(a8, b8, scale)
     got = _run_fast(sg, a8, b8, scale)

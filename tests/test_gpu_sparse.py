@@ -1,4 +1,4 @@
-"""GPU parity of the 2:4 structured-sparse FP8 GEMM (BASELINE config 5) through the C ABI.
+"""GPU parity of the 2:4 structured-sparse FP8 GEMM (benchmark configuration 5) through the C ABI.
 
 The oracle's sparse GEMM is its dense GEMM on the decompressed weights, and the compressed
 format is pinned on the CPU by tests/test_oracle_gemm.py; here the HIP kernel, which feeds
@@ -91,7 +91,7 @@ def test_sparse_tuned_configs(sg, oracle, cfg, shape):
 @pytest.mark.parametrize("n,k", [(4096, 14336), (14336, 4096)])
 @pytest.mark.parametrize("m", [1, 8, 16, 32])
 def test_config5_shapes(sg, oracle, m, n, k):
-    """BASELINE config 5 at full size: prune N(0,1) 2:4, quantise the pruned tensor, compress."""
+    """benchmark configuration 5 at full size: prune N(0,1) 2:4, quantise the pruned tensor, compress."""
     a8, vals, meta, b8, scale = oracle.make_sparse24_operands(m, n, k, seed=0)
     assert vals.shape == (n, k // 2) and meta.shape == (n, k // 8)
     ref = oracle.gemm_sparse24(a8, vals, meta, scale)

@@ -1,4 +1,4 @@
-"""The process / stdout protocol of the reference's drivers (SURVEY level-2 boundary):
+"""The process / stdout protocol of the reference's drivers (the process-level boundary):
 parsing rules on the CPU, the real mains on the GPU."""
 import os
 import subprocess

@@ -134,7 +134,7 @@ def test_b_stride_and_transposition(oracle):
 
 
 def test_config1_against_torch_fp64(oracle):
-    """BASELINE config 1 (8 x 4096 x 4096, seed 0): oracle vs torch fp64 matmul of the dequantised operands."""
+    """benchmark configuration 1 (8 x 4096 x 4096, seed 0): oracle vs torch fp64 matmul of the dequantised operands."""
     a8, b8, scale = oracle.make_gemm_operands(8, 4096, 4096, seed=0)
     truth = torch.from_numpy(_dec(a8)) @ torch.from_numpy(_dec(b8)).T * float(scale)
     got = oracle.bf16_to_f32(oracle.gemm_omp(a8, b8, scale))
