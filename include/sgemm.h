@@ -126,7 +126,8 @@ typedef struct SgTuning {
     int persistent_wgs_per_cu; /* LDS ring: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU */
     int wave_tiles;    /* LDS ring: 1 = every wavefront owns whole tiles over the full K range and the activations
                           stay resident in LDS; 2 = persistent K-split workgroups with resident activations
-                          (both need persistent_wgs_per_cu >= 1, split_k = 1, m <= 16*m_blocks); + 4 = persistent
+                          3 = the same with the activations in the wavefronts' registers (k = 256 * waves * 1, 2 or 4)
+                          (all need persistent_wgs_per_cu >= 1, split_k = 1, m <= 16*m_blocks); + 4 = persistent
                           workgroups get one extra wavefront that streams nothing and does every reduction and store */
 } SgTuning;
 

@@ -101,6 +101,7 @@ struct Config {
     int persist;  // LDS engine: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU walking the tiles
     int wavetile; // LDS engine, bits 0-1: 1 = every wave owns whole tiles, activations resident in LDS (persist = workgroups per CU);
                   //             2 = persistent K-split workgroups with the activations resident in LDS
+                  //             3 = ... resident in the waves' registers (k = 256 * waves * {1, 2, 4});  bit 2: epilogue wave
 };
 
 static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out) {
@@ -167,6 +168,22 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         const size_t cap = (size_t)dev->cu_count * c.persist;
         if (want > cap) want = cap;
         grid = (unsigned)want;
+    } else if (c.persist > 0 && (c.wavetile & 3) == 3) {
+        // activations resident in registers: every wave keeps the fragments of its own K blocks
+        if (c.split_k != 1 || a.m_tiles != 1) return SG_INVALID_CONFIG;
+        const int blocks = a.k / 256;
+        if (blocks % c.waves != 0) return SG_INVALID_CONFIG;
+        const int pt = blocks / c.waves;
+        if (pt * c.mt > 4) return SG_INVALID_CONFIG;
+        DeviceInfo* dev;
+        if (int rc = get_device_info(&dev)) return rc;
+        const size_t want = (size_t)dev->cu_count * c.persist;
+        if (want < grid) grid = (unsigned)want;
+        const unsigned threads = (unsigned)(c.waves + ((c.wavetile & 4) ? 1 : 0)) * 64;
+        if (threads > 1024) return SG_TOO_MANY_WARPS;
+        const size_t lds_x = (size_t)c.waves * c.depth * c.rg * 4096 + 2u * c.waves * c.rg * c.mt * 1024;
+        if (lds_x > 159 * 1024) return SG_INVALID_CONFIG;
+        return launch_xreg(c.mt, c.rg, pt, c.depth, a, grid, threads, lds_x, stream);
     } else if (c.persist > 0) {
         if (c.split_k != 1) return SG_INVALID_CONFIG;
         mode = 1;
@@ -436,6 +453,13 @@ static Config pick_config(int m, int n, int k, int cu_count) {
                 return c;
             }
             c.waves = m <= 8 ? 8 : 6;
+            if (c.mt == 2 && blocks % 8 == 0 && (blocks / 8) * c.mt <= 4) {
+                // 17..32 rows and a short K: eight waves keep the activation fragments of their own K blocks in registers
+                c.waves = 8;
+                c.depth = 3;
+                c.wavetile = 3;
+                return c;
+            }
             if (c.mt == 2) {                    // wide tiles share one activation stage among four weight tiles
                 c.persist = 0;
                 c.rg = 4;

@@ -39,4 +39,15 @@ __device__ __forceinline__ i64x2 load16_stream(const void* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const i64x2*>(p));
 }
 
+// Workgroups are dispatched round-robin over the 8 XCDs (workgroup b runs on XCD b % 8), each with its own
+// L2.  A 16-row tile writes only 32 bytes of every output row, so the four tiles that share a 128-byte line of
+// D should pass through the same L2, which then merges them before they reach memory: workgroup b is given
+// position xcd_order(b) in tile order, where all workgroups of one XCD are neighbours.
+constexpr int kXcds = 8;
+__device__ __forceinline__ int xcd_order(int b, int groups) {
+    const int x = b % kXcds, i = b / kXcds;
+    const int q = groups / kXcds, rem = groups % kXcds;
+    return x * q + (x < rem ? x : rem) + i;
+}
+
 }  // namespace sg

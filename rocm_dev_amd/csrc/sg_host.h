@@ -38,6 +38,9 @@ int SG_RING_LAUNCHER(1)(int bl, int xu, int nt, const RingArgs& ra, unsigned gri
 int SG_RING_LAUNCHER(2)(int bl, int xu, int nt, const RingArgs& ra, unsigned grid, unsigned threads, size_t lds,
                         hipStream_t stream);
 
+// persistent LDS ring with the activations resident in registers: pt K blocks per wave and tile
+int launch_xreg(int mt, int rg, int pt, int depth, const StreamArgs& a, unsigned grid, unsigned threads, size_t lds,
+                hipStream_t stream);
 int launch_mid(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream);
 
 struct SparseArgs;

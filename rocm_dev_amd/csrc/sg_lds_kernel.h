@@ -106,6 +106,14 @@ __device__ __forceinline__ void mma_block_256(const uint8_t* w, const uint8_t* x
         }
 }
 
+// Tiles of a persistent workgroup: one contiguous run (not a stride of gridDim.x), runs in XCD order.
+struct TileRun { int first, count; };
+__device__ __forceinline__ TileRun persistent_tile_run(int total_tiles) {
+    const int groups = (int)gridDim.x, b = xcd_order((int)blockIdx.x, (int)gridDim.x);
+    const int q = total_tiles / groups, rem = total_tiles % groups;
+    return TileRun{b * q + (b < rem ? b : rem), q + (b < rem ? 1 : 0)};
+}
+
 constexpr int lds_stage_bytes(int RG, int XU) { return (RG * 4 + XU) * 1024; }
 // Eight or more accumulator fragments per wave need more than the 128 VGPRs a 16-wave workgroup
 // leaves each wave; those instantiations accept at most 8 waves per workgroup.
@@ -129,7 +137,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     const int wave = wave_id();
     const int waves = a.waves;
 
-    int bid = blockIdx.x;
+    int bid = xcd_order((int)blockIdx.x, (int)gridDim.x);
     const int tile_n = bid % a.n_tiles;
     bid /= a.n_tiles;
     const int split = bid % a.split_k;
@@ -248,7 +256,8 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     const int r = lane & 15, g = lane >> 4;
 
     const int total_tiles = a.n_tiles * a.m_tiles;
-    const int my_tiles = ((int)blockIdx.x < total_tiles) ? (total_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    const TileRun run = persistent_tile_run(total_tiles);
+    const int my_tiles = run.count;
     const int blocks = a.k >> 8;
     // a workgroup launched with one wave more than a.waves has a dedicated epilogue wave: it
     // streams nothing and does every reduction and store, so that the streaming waves never have
@@ -268,7 +277,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     f32x4* red = reinterpret_cast<f32x4*>(ring + x_bytes + (size_t)waves * (DEPTH * STAGE_BYTES));
 
     auto tile_origin = [&](int j, int& m0, int& n0) __attribute__((always_inline)) {  // j-th tile of this workgroup
-        const int t = (int)blockIdx.x + j * (int)gridDim.x;
+        const int t = run.first + j;
         n0 = (t % a.n_tiles) * (16 * RG);
         m0 = (t / a.n_tiles) * (16 * MT);
     };

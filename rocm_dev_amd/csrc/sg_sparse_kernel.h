@@ -54,7 +54,7 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
     const int wave = wave_id();
     const int waves = a.waves;
 
-    int bid = blockIdx.x;
+    int bid = xcd_order((int)blockIdx.x, (int)gridDim.x);
     const int tile_n = bid % a.n_tiles;
     bid /= a.n_tiles;
     const int split = bid % a.split_k;

@@ -94,7 +94,7 @@ stream_gemm_kernel(const StreamArgs a) {
     const int waves = a.waves;
     const int r = lane & 15, g = lane >> 4;
 
-    int bid = blockIdx.x;
+    int bid = xcd_order((int)blockIdx.x, (int)gridDim.x);
     const int tile_n = bid % a.n_tiles;
     bid /= a.n_tiles;
     const int split = bid % a.split_k;

@@ -212,6 +212,49 @@ def test_lds_ring_persistent(sg, oracle, cfg, shape):
             assert np.array_equal(bits(D4), got)
 
 
+XREG_CONFIGS = [
+    # waves, row_tiles, depth, epilogue wave
+    (8, 1, 2, True),
+    (8, 1, 3, False),
+    (4, 2, 2, True),
+    (16, 1, 2, False),
+    (8, 2, 4, True),
+    (4, 1, 3, True),
+    (2, 1, 2, False),
+]
+
+
+@pytest.mark.parametrize("cfg", XREG_CONFIGS)
+@pytest.mark.parametrize("shape", [(8, 28672, 4096), (32, 6144, 4096), (16, 4100, 2048), (5, 9000, 1024), (27, 130, 4096),
+                                   (1, 512, 512), (32, 2048, 2048)])
+def test_lds_ring_activations_in_registers(sg, oracle, cfg, shape):
+    """Persistent workgroups whose waves keep the activation fragments of their own K blocks in registers
+    (k must be 256 * waves * {1, 2, 4}, at most four fragments per wave)."""
+    waves, row_tiles, depth, epi = cfg
+    m, n, k = shape
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=12)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kw = dict(engine=2, waves=waves, row_tiles=row_tiles, depth=depth, persistent_wgs_per_cu=1, wave_tiles=3 + (4 if epi else 0))
+    rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
+    torch.cuda.synchronize()
+    blocks = k // 256
+    fits = blocks % waves == 0 and (blocks // waves) in (1, 2, 4) and (blocks // waves) * (1 if m <= 16 else 2) <= 4
+    if rc == 6:
+        assert not fits or depth * row_tiles * waves * 4 > 140 or waves + epi > 8, "a configuration that fits was rejected"
+        pytest.skip("configuration does not apply to this shape")
+    assert rc == 0, sg.strerror(rc)
+    got = bits(D)
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
+    # same partial sums in the same order as the persistent kernel with the activations in the stage
+    D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kw["wave_tiles"] = 0
+    if sg.skinny_gemm_tuned(A, B, D2, S, **kw) == 0:
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(D2), got)
+
+
 RING_CONFIGS = [
     # A_producers, B_producers, consumers, b_lanes, qsize
     (1, 1, 1, 1, 1),
