@@ -32,7 +32,7 @@ COLD_BYTES = 640e6          # per shape: distinct weight bytes cycled through (>
 # HBM bytes per launch of the dominant kernel (gate_up, M = 8), measured off-line with two
 # rocprofv3 --pmc runs (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0, factors from a 256 MiB copy);
 # the runs and their arithmetic are in profiles/dense_gemm_decode_step_m8_pmc_traffic.md
-RECORDED_TRAFFIC = {("gate_up", 8): 118323244}
+RECORDED_TRAFFIC = {("gate_up", 8): 118372433}
 
 
 def gemm_bytes(m, n, k):

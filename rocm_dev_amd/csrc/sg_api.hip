@@ -446,7 +446,7 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             c.rg = 1;
             c.persist = 1;
             const size_t x_res = (size_t)blocks * xu0 * 1024;
-            c.waves = m <= 8 ? 8 : 7;
+            c.waves = 8;
             c.depth = 2;
             if (m <= 16 * c.mt && x_res + (size_t)c.waves * (c.depth * 4 + 2 * c.mt) * 1024 + 4096 <= 159 * 1024) {
                 c.wavetile = 2 | 4;   // resident activations + a dedicated epilogue wave (0.3-0.9 us on gate_up)
