@@ -233,8 +233,8 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
 }
 
 // ---------------------------------------------------------------------------------------------
-// Persistent variant for shapes with many more tiles than CUs.  A workgroup walks tiles
-// blockIdx.x, blockIdx.x + gridDim.x, ... and every wave's ring simply continues across the
+// Persistent variant for shapes with many more tiles than CUs.  A workgroup walks a contiguous
+// run of tiles (persistent_tile_run) and every wave's ring simply continues across the
 // tile boundary: while the waves meet to reduce and store tile j, the DMAs of tile j+1 are
 // already in flight, so HBM never sees the ramp-down / ramp-up of a workgroup hand-over.
 // (The reference's kernel is persistent for the same reason: skinny_gemm_kernel.cu:44-51.)
