@@ -138,6 +138,31 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const
  * out[8] = {split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops}. */
 int sg_skinny_gemm_pick(int m, int n, int k, int out[8]);
 
+/* The complete record sg_skinny_gemm_auto would launch for the shape: the tuning table's entry when
+ * there is one (*from_table = 1), the built-in heuristics' otherwise (0).  from_table may be NULL. */
+int sg_skinny_gemm_choice(int m, int n, int k, SgTuning* out, int* from_table);
+
+/* Per-shape tuning table - the run-time form of what the reference's grid search produces: there the
+ * best #define set found by grid.py (:84-145, search space :151-159) is pasted into core.cu and picked
+ * by the 249-arm macro chain of skinny_gemm_caller.cu:86-334; here a tuning driver stores the best
+ * SgTuning per (m, n, k) and sg_skinny_gemm_auto / _fastpath / _rowcol use it instead of the built-in
+ * heuristics.  A record the kernels cannot run for the shape (no such instantiation, ring larger than
+ * LDS, ...) is skipped at launch and the heuristics' choice runs.  The table is process-wide and may be
+ * read and changed from any thread; a launch uses the table as it is when the launch is made.
+ *   sg_tuning_set    stores a copy of *t for the shape (engine 1, 2 or 4); t == NULL removes the entry
+ *   sg_tuning_get    SG_SUCCESS and *out, or SG_INVALID_CONFIG when the table has no entry
+ *   sg_tuning_load   merges a file into the table; SG_BAD_ARGUMENT (table unchanged) if the file cannot be
+ *                    read or any line is malformed.  Format: first line "sgemm-tuning 1", then one record
+ *                    per line as thirteen integers "m n k engine split_k waves row_tiles m_blocks depth
+ *                    k_chunks non_temporal persistent_wgs_per_cu wave_tiles"; '#' starts a comment
+ *   sg_tuning_save   writes the whole table in that format */
+int sg_tuning_set(int m, int n, int k, const SgTuning* t);
+int sg_tuning_get(int m, int n, int k, SgTuning* out);
+int sg_tuning_count(void);
+int sg_tuning_clear(void);
+int sg_tuning_load(const char* path);
+int sg_tuning_save(const char* path);
+
 /* Replaces  template<class out> void async_gemm(const fp8* A, const fp8* B, out* D, int m,
  * int n, int k)  (async_gemm_sparse/sparse_k.cu:45-69, async_gemm_blanes/sparse_k.cu,
  * async_gemm_16x16x64/src.cu:55-82): D = A * B^T without a scale, default stream, through

@@ -17,10 +17,17 @@ from .api import (  # noqa: F401
     sparse24_gemm,
     SgTuning,
     skinny_gemm_fastpath,
+    skinny_gemm_choice,
     skinny_gemm_pick,
     skinny_gemm_rowcol,
     skinny_gemm_tuned,
     strerror,
     tiled_sum_reduce,
+    tuning_clear,
+    tuning_count,
+    tuning_get,
+    tuning_load,
+    tuning_save,
+    tuning_set,
 )
 from .build import build  # noqa: F401

@@ -26,6 +26,13 @@ SIGNATURES = {
     "sg_skinny_gemm_rowcol": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm_tuned": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sg_skinny_gemm_pick": (_i, [_i, _i, _i, C.POINTER(_i * 8)]),
+    "sg_skinny_gemm_choice": (_i, [_i, _i, _i, _vp, C.POINTER(_i)]),
+    "sg_tuning_set": (_i, [_i, _i, _i, _vp]),
+    "sg_tuning_get": (_i, [_i, _i, _i, _vp]),
+    "sg_tuning_count": (_i, []),
+    "sg_tuning_clear": (_i, []),
+    "sg_tuning_load": (_i, [C.c_char_p]),
+    "sg_tuning_save": (_i, [C.c_char_p]),
     "sg_async_gemm_f32": (_i, [_vp, _vp, _vp, _i, _i, _i]),
     "sg_async_gemm_bf16": (_i, [_vp, _vp, _vp, _i, _i, _i]),
     "sg_sparse24_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),

@@ -96,7 +96,12 @@ class SgTuning(C.Structure):
                  "persistent_wgs_per_cu", "wave_tiles")]
 
 
-ENGINE_AUTO, ENGINE_DIRECT, ENGINE_LDS = 0, 1, 2
+ENGINE_AUTO, ENGINE_DIRECT, ENGINE_LDS, ENGINE_MID = 0, 1, 2, 4
+TUNING_FIELDS = tuple(name for name, _ in SgTuning._fields_)
+
+
+def tuning_as_dict(t):
+    return {name: getattr(t, name) for name in TUNING_FIELDS}
 
 
 def skinny_gemm_rowcol(A, B, D, scale_tensor=None, row_scales=None, col_scales=None, check=False):
@@ -138,6 +143,44 @@ def skinny_gemm_pick(m, n, k):
         raise SgError(rc)
     names = ("split_k", "A_producers", "B_producers", "consumers", "b_lanes", "qsize", "op_m", "ops")
     return dict(zip(names, list(out)))
+
+
+def skinny_gemm_choice(m, n, k):
+    """(record, from_table): the complete SgTuning the fastpath would launch for the shape, and whether it comes
+    from the tuning table rather than the built-in heuristics."""
+    t, from_table = SgTuning(), C.c_int(0)
+    rc = lib.sg_skinny_gemm_choice(m, n, k, C.byref(t), C.byref(from_table))
+    if rc != 0:
+        raise SgError(rc)
+    return t, bool(from_table.value)
+
+
+def tuning_set(m, n, k, tuning):
+    """Store `tuning` (an SgTuning, or None to remove the entry) as the record the fastpath uses for the shape."""
+    return _done(lib.sg_tuning_set(m, n, k, None if tuning is None else C.byref(tuning)), True)
+
+
+def tuning_get(m, n, k):
+    """The table's SgTuning for the shape, or None."""
+    t = SgTuning()
+    return t if lib.sg_tuning_get(m, n, k, C.byref(t)) == 0 else None
+
+
+def tuning_count():
+    return lib.sg_tuning_count()
+
+
+def tuning_clear():
+    return _done(lib.sg_tuning_clear(), True)
+
+
+def tuning_load(path):
+    """Merge a tuning file (written by tuning_save or rocm_dev_amd.autotune) into the table."""
+    return _done(lib.sg_tuning_load(str(path).encode()), True)
+
+
+def tuning_save(path):
+    return _done(lib.sg_tuning_save(str(path).encode()), True)
 
 
 class HFRK_skinny_gemm:

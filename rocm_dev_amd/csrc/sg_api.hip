@@ -1,8 +1,12 @@
 // C ABI of libsgemm.so: argument validation, configuration choice and launches.
 // The contract of every entry point is documented in include/sgemm.h.
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
+#include <map>
 #include <mutex>
+#include <tuple>
 
 #include "sg_host.h"
 #include "sg_stream_kernel.h"
@@ -518,6 +522,61 @@ static Config pick_config(int m, int n, int k, int cu_count) {
     return c;
 }
 
+static Config config_from_tuning(const SgTuning& t) {
+    Config c;
+    c.engine = t.engine;
+    c.mt = t.m_blocks;
+    c.rg = t.row_tiles;
+    c.ku = t.k_chunks;
+    c.depth = t.depth;
+    c.waves = t.waves;
+    c.split_k = t.split_k;
+    c.nt = t.non_temporal;
+    c.persist = t.persistent_wgs_per_cu;
+    c.wavetile = t.wave_tiles;
+    return c;
+}
+
+static Config heuristic_config(int m, int n, int k, int cu_count) {
+    return (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, cu_count) : pick_config(m, n, k, cu_count);
+}
+
+// ---- per-shape tuning table ---------------------------------------------------------------
+// What a tuning driver measured to be the best record for a shape; consulted before the
+// heuristics by the launchers that choose their own configuration.  Process-wide, any thread.
+static std::mutex g_table_mutex;
+static std::map<std::tuple<int, int, int>, SgTuning> g_table;
+static std::atomic<int> g_table_entries{0};   // an empty table costs the launch path one relaxed load
+
+static bool table_lookup(int m, int n, int k, SgTuning* out) {
+    if (g_table_entries.load(std::memory_order_relaxed) == 0) return false;
+    std::lock_guard<std::mutex> lock(g_table_mutex);
+    const auto it = g_table.find(std::make_tuple(m, n, k));
+    if (it == g_table.end()) return false;
+    *out = it->second;
+    return true;
+}
+
+// A record is rejected by the launch functions before anything is enqueued with one of these codes
+// (no kernel for it, ring does not fit LDS, k not a multiple of the engine's stage, ...).
+static bool rejected_before_launch(int rc) {
+    return rc == SG_INVALID_CONFIG || rc == SG_K_NOT_DIVISIBLE_BY_WARPTILE_K || rc == SG_TOO_MANY_WARPS ||
+           rc == SG_WORKSPACE_TOO_SMALL;
+}
+
+// The table's record for the shape if it has a usable one, the heuristics' otherwise.
+static int launch_chosen(const StreamArgs& a, int cu_count, hipStream_t stream) {
+    SgTuning t;
+    if (table_lookup(a.m, a.n, a.k, &t) && t.engine != ENGINE_AUTO) {
+        const Config c = config_from_tuning(t);
+        if (c.engine == ENGINE_MID || c.mt == 1 || c.mt == 2) {
+            const int rc = launch_config(c, a, stream);
+            if (!rejected_before_launch(rc)) return rc;
+        }
+    }
+    return launch_config(heuristic_config(a.m, a.n, a.k, cu_count), a, stream);
+}
+
 }  // namespace sg
 
 using namespace sg;
@@ -622,19 +681,8 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D, const floa
     if (!scale_tensor) return SG_BAD_ARGUMENT;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    Config c;
-    c.engine = t->engine;
-    c.mt = t->m_blocks;
-    c.rg = t->row_tiles;
-    c.ku = t->k_chunks;
-    c.depth = t->depth;
-    c.waves = t->waves;
-    c.split_k = t->split_k;
-    c.nt = t->non_temporal;
-    c.persist = t->persistent_wgs_per_cu;
-    c.wavetile = t->wave_tiles;
-    if (c.engine == ENGINE_AUTO)
-        c = (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, dev->cu_count) : pick_config(m, n, k, dev->cu_count);
+    Config c = config_from_tuning(*t);
+    if (c.engine == ENGINE_AUTO) c = heuristic_config(m, n, k, dev->cu_count);
     if (c.engine != ENGINE_MID && c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
@@ -655,6 +703,23 @@ int sg_skinny_gemm_pick(int m, int n, int k, int out[8]) {
     return SG_SUCCESS;
 }
 
+int sg_skinny_gemm_choice(int m, int n, int k, SgTuning* out, int* from_table) {
+    if (!out || m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
+    if (table_lookup(m, n, k, out)) {
+        if (from_table) *from_table = 1;
+        return SG_SUCCESS;
+    }
+    DeviceInfo* dev;
+    int cu = 256;
+    if (get_device_info(&dev) == SG_SUCCESS) cu = dev->cu_count;
+    const Config c = heuristic_config(m, n, k, cu);
+    out->engine = c.engine; out->split_k = c.split_k; out->waves = c.waves; out->row_tiles = c.rg; out->m_blocks = c.mt;
+    out->depth = c.depth; out->k_chunks = c.ku; out->non_temporal = c.nt; out->persistent_wgs_per_cu = c.persist;
+    out->wave_tiles = c.wavetile;
+    if (from_table) *from_table = 0;
+    return SG_SUCCESS;
+}
+
 int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,
                         int b_stride, void* stream) {
     if (n % 2 != 0) return SG_N_NOT_EVEN;
@@ -663,12 +728,11 @@ int sg_skinny_gemm_auto(const uint8_t* A, const uint8_t* B, void* D, const float
     if (!scale_tensor) return SG_BAD_ARGUMENT;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const Config c = (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, dev->cu_count) : pick_config(m, n, k, dev->cu_count);
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
     a.out_f32 = 0;
-    return launch_config(c, a, static_cast<hipStream_t>(stream));
+    return launch_chosen(a, dev->cu_count, static_cast<hipStream_t>(stream));
 }
 
 int sg_skinny_gemm_rowcol(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, const float* row_scales,
@@ -679,14 +743,103 @@ int sg_skinny_gemm_rowcol(const uint8_t* A, const uint8_t* B, void* D, const flo
     if ((reinterpret_cast<uintptr_t>(row_scales) | reinterpret_cast<uintptr_t>(col_scales)) & 3u) return SG_BAD_ALIGNMENT;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const Config c = (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, dev->cu_count) : pick_config(m, n, k, dev->cu_count);
     StreamArgs a{};
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;   // nullptr = 1.0f
     a.row_scale = row_scales;
     a.col_scale = col_scales;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
     a.out_f32 = 0;
-    return launch_config(c, a, static_cast<hipStream_t>(stream));
+    return launch_chosen(a, dev->cu_count, static_cast<hipStream_t>(stream));
+}
+
+int sg_tuning_set(int m, int n, int k, const SgTuning* t) {
+    if (m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
+    std::lock_guard<std::mutex> lock(g_table_mutex);
+    if (t) {
+        if (t->engine != ENGINE_DIRECT && t->engine != ENGINE_LDS && t->engine != ENGINE_MID) return SG_INVALID_CONFIG;
+        g_table[std::make_tuple(m, n, k)] = *t;
+    } else {
+        g_table.erase(std::make_tuple(m, n, k));
+    }
+    g_table_entries.store((int)g_table.size(), std::memory_order_relaxed);
+    return SG_SUCCESS;
+}
+
+int sg_tuning_get(int m, int n, int k, SgTuning* out) {
+    if (!out) return SG_BAD_ARGUMENT;
+    return table_lookup(m, n, k, out) ? SG_SUCCESS : SG_INVALID_CONFIG;
+}
+
+int sg_tuning_count(void) { return g_table_entries.load(std::memory_order_relaxed); }
+
+int sg_tuning_clear(void) {
+    std::lock_guard<std::mutex> lock(g_table_mutex);
+    g_table.clear();
+    g_table_entries.store(0, std::memory_order_relaxed);
+    return SG_SUCCESS;
+}
+
+// File: first line "sgemm-tuning 1"; then one record per line, thirteen integers
+//   m n k engine split_k waves row_tiles m_blocks depth k_chunks non_temporal persistent_wgs_per_cu wave_tiles
+// '#' starts a comment; blank lines are skipped.
+int sg_tuning_load(const char* path) {
+    if (!path) return SG_BAD_ARGUMENT;
+    FILE* f = std::fopen(path, "r");
+    if (!f) return SG_BAD_ARGUMENT;
+    std::map<std::tuple<int, int, int>, SgTuning> parsed;
+    char line[512];
+    bool header = false, ok = true;
+    while (ok && std::fgets(line, sizeof line, f)) {
+        char* hash = std::strchr(line, '#');
+        if (hash) *hash = 0;
+        char* p = line;
+        while (*p == ' ' || *p == '\t' || *p == '\r' || *p == '\n') p++;
+        if (!*p) continue;
+        if (!header) {
+            int version = 0;
+            char tail = 0;
+            ok = std::sscanf(p, "sgemm-tuning %d %c", &version, &tail) == 1 && version == 1;
+            header = true;
+            continue;
+        }
+        int v[13];
+        char tail = 0;
+        const int got = std::sscanf(p, "%d %d %d %d %d %d %d %d %d %d %d %d %d %c", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5],
+                                    &v[6], &v[7], &v[8], &v[9], &v[10], &v[11], &v[12], &tail);
+        if (got != 13 || v[0] <= 0 || v[1] <= 0 || v[2] <= 0 ||
+            (v[3] != ENGINE_DIRECT && v[3] != ENGINE_LDS && v[3] != ENGINE_MID)) {
+            ok = false;
+            break;
+        }
+        SgTuning t;
+        t.engine = v[3]; t.split_k = v[4]; t.waves = v[5]; t.row_tiles = v[6]; t.m_blocks = v[7]; t.depth = v[8];
+        t.k_chunks = v[9]; t.non_temporal = v[10]; t.persistent_wgs_per_cu = v[11]; t.wave_tiles = v[12];
+        parsed[std::make_tuple(v[0], v[1], v[2])] = t;
+    }
+    std::fclose(f);
+    if (!ok || !header) return SG_BAD_ARGUMENT;   // the table is left as it was
+    std::lock_guard<std::mutex> lock(g_table_mutex);
+    for (const auto& e : parsed) g_table[e.first] = e.second;
+    g_table_entries.store((int)g_table.size(), std::memory_order_relaxed);
+    return SG_SUCCESS;
+}
+
+int sg_tuning_save(const char* path) {
+    if (!path) return SG_BAD_ARGUMENT;
+    FILE* f = std::fopen(path, "w");
+    if (!f) return SG_BAD_ARGUMENT;
+    std::fprintf(f, "sgemm-tuning 1\n# m n k engine split_k waves row_tiles m_blocks depth k_chunks non_temporal "
+                    "persistent_wgs_per_cu wave_tiles\n");
+    {
+        std::lock_guard<std::mutex> lock(g_table_mutex);
+        for (const auto& e : g_table) {
+            const SgTuning& t = e.second;
+            std::fprintf(f, "%d %d %d %d %d %d %d %d %d %d %d %d %d\n", std::get<0>(e.first), std::get<1>(e.first),
+                         std::get<2>(e.first), t.engine, t.split_k, t.waves, t.row_tiles, t.m_blocks, t.depth, t.k_chunks,
+                         t.non_temporal, t.persistent_wgs_per_cu, t.wave_tiles);
+        }
+    }
+    return std::fclose(f) == 0 ? SG_SUCCESS : SG_BAD_ARGUMENT;
 }
 
 int sg_skinny_gemm_fastpath(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n,

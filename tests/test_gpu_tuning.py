@@ -1,0 +1,112 @@
+"""GPU side of the per-shape tuning table and the grid-search driver (run-time counterpart of the
+reference's grid.py:84-159): a stored record is what the fastpath launches, an unusable record falls
+back to the heuristics, and the driver's winners are records whose results pass the GEMM parity bar."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import bits, dev, gemm_tol, scale_tensor
+from rocm_dev_amd import autotune
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture()
+def sg():
+    import rocm_dev_amd
+    rocm_dev_amd.tuning_clear()
+    yield rocm_dev_amd
+    rocm_dev_amd.tuning_clear()
+
+
+def _record(sg, r):
+    return sg.SgTuning(*(r[f] for f in autotune.FIELDS))
+
+
+def _fast(sg, A, B, S, m, n):
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = sg.skinny_gemm_fastpath(A, B, D, S)
+    torch.cuda.synchronize()
+    assert rc == 0, sg.strerror(rc)
+    return bits(D)
+
+
+def _tuned(sg, A, B, S, m, n, r):
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = sg.skinny_gemm_tuned(A, B, D, S, **r)
+    torch.cuda.synchronize()
+    assert rc == 0, sg.strerror(rc)
+    return bits(D)
+
+
+@pytest.mark.parametrize("shape,rec", [
+    ((8, 4096, 4096), autotune.record(1, 2, 4, 2, 1, 2, 2)),              # direct engine, split-K 2
+    ((8, 4096, 4096), autotune.record(2, 1, 3, 2, 1, 3, 4, 1, 0, 0)),      # LDS ring, three waves
+    ((32, 6144, 4096), autotune.record(2, 1, 8, 1, 2, 3, 4, 1, 1, 3)),     # activations in registers
+    ((128, 1024, 2048), autotune.record(4, 1, 8, 2, 2, 4, 2)),             # mid-batch, shallow activation ring
+])
+def test_fastpath_launches_the_stored_record(sg, oracle, shape, rec):
+    m, n, k = shape
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=5)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    before = _fast(sg, A, B, S, m, n)
+    explicit = _tuned(sg, A, B, S, m, n, rec)
+    assert oracle.max_rel_err_bf16(explicit, ref) <= gemm_tol(k)
+    sg.tuning_set(m, n, k, _record(sg, rec))
+    choice, from_table = sg.skinny_gemm_choice(m, n, k)
+    assert from_table and {f: getattr(choice, f) for f in autotune.FIELDS} == rec
+    after = _fast(sg, A, B, S, m, n)
+    # every reduction in the library has a fixed order, so the same record gives the same bits
+    assert np.array_equal(after, explicit)
+    assert oracle.max_rel_err_bf16(after, ref) <= gemm_tol(k)
+    # the row/column-scaled entry point goes through the same choice
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_rowcol(A, B, D, S) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(D), explicit)
+    sg.tuning_set(m, n, k, None)
+    assert np.array_equal(_fast(sg, A, B, S, m, n), before)
+
+
+@pytest.mark.parametrize("rec", [
+    autotune.record(2, 1, 16, 4, 1, 8),                 # ring far larger than LDS
+    autotune.record(2, 1, 4, 3, 1, 2),                  # no LDS-ring kernel with three row tiles
+    autotune.record(4, 1, 8, 4, 8, 3, 2),               # a mid-batch record stored for a skinny shape
+    autotune.record(2, 1, 7, 1, 1, 3, 4, 1, 1, 3),      # registers variant needs k = 256 * waves * {1, 2, 4}
+])
+def test_unusable_record_falls_back(sg, oracle, rec):
+    m, n, k = 8, 1024, 4096
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=6)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    before = _fast(sg, A, B, S, m, n)
+    D = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+    rc = sg.skinny_gemm_tuned(A, B, D, S, **rec)
+    if rec["engine"] != 4:                              # (mid-batch kernels do run small m; just not the table's job)
+        assert rc != 0
+    sg.tuning_set(m, n, k, _record(sg, rec))
+    after = _fast(sg, A, B, S, m, n)
+    if rc != 0:
+        assert np.array_equal(after, before)
+    assert oracle.max_rel_err_bf16(after, oracle.gemm_omp(a8, b8, scale)) <= gemm_tol(k)
+
+
+def test_driver_measures_checks_and_writes_a_loadable_table(sg, oracle, tmp_path, capsys):
+    m, n, k = 8, 2048, 1024
+    kept, base_us, ran = autotune.tune_shape(m, n, k, top=3, launches=8, limit=40)
+    assert ran > 10 and 1 <= len(kept) <= 3 and base_us > 0
+    assert [us for us, _ in kept] == sorted(us for us, _ in kept)
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=7)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    for us, rec in kept:
+        assert rec in autotune.search_space(m, n, k) and 0 < us < 1e4
+        assert oracle.max_rel_err_bf16(_tuned(sg, A, B, S, m, n, rec), ref) <= gemm_tol(k)
+    out = tmp_path / "tuning.txt"
+    assert autotune.main(["--shapes", "%dx%dx%d" % (m, n, k), "64x512x1024", "--out", str(out), "--launches", "8",
+                          "--limit", "24", "--min-gain", "-1"]) == 0          # -1: always keep the winner
+    entries = autotune.parse_table(out.read_text())
+    assert set(entries) == {(m, n, k), (64, 512, 1024)} and entries[(64, 512, 1024)]["engine"] == 4
+    sg.tuning_load(out)
+    assert sg.tuning_count() == 2
+    assert oracle.max_rel_err_bf16(_fast(sg, A, B, S, m, n), ref) <= gemm_tol(k)
