@@ -261,7 +261,7 @@ static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
 }
 
 // Mid-batch engine: c.rg = 16-row weight fragments per wave (2 or 4), c.mt = 16-row activation
-// fragments per wave (2, 4 or 8); a workgroup tile is 32*c.rg weight rows x 32*c.mt activation rows.
+// fragments per wave (2, 4 or 8); a workgroup tile is 16*c.rg*(waves/2) weight rows x 32*c.mt activation rows.
 static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) {
     if (a.k % 128 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if ((c.rg != 2 && c.rg != 4) || (c.mt != 2 && c.mt != 4 && c.mt != 8) || c.depth < 2) return SG_INVALID_CONFIG;
