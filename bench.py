@@ -54,6 +54,10 @@ def main():
     ap.add_argument("--mid-batch-counters", action="store_true",
                     help="only launch the mid-batch GEMMs (M = 64, 128, 256), eagerly, three times each, and exit "
                          "(for MFMA-utilisation counter runs; prints no JSON line)")
+    ap.add_argument("--decode-counters", action="store_true",
+                    help="only launch the decode-sweep GEMMs (four projection shapes x M = 1, 8, 32), eagerly, three "
+                         "times each on cold weights, after three 256 MiB copies of known traffic, and exit "
+                         "(for HBM-traffic counter runs; prints no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1")
@@ -68,6 +72,28 @@ def main():
     torch.manual_seed(0)
     if lib.sg_init() != 0:
         sys.exit("bench.py: sg_init failed")
+
+    if args.decode_counters:
+        one = torch.ones(1, device="cuda")
+        src = torch.empty(256 << 20, device="cuda", dtype=torch.uint8)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        for name, (n, k) in SHAPES.items():
+            copies = max(3, int(COLD_BYTES // (n * k)) + 1)
+            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(copies)]
+            for m in (1, 8, 32):
+                a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+                d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+                for i in range(3):
+                    w = wb[(3 * (m % 5) + i) % copies]
+                    rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), w.data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, None)
+                    if rc != 0:
+                        raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
+                torch.cuda.synchronize()
+            del wb
+        return
 
     if args.mid_batch_counters:
         one = torch.ones(1, device="cuda")
