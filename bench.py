@@ -368,6 +368,18 @@ def main():
                "kind": "port", "sample": "one full step (4 GEMMs, M=%d) with the oracle's OpenMP loop: %.3f s; "
                "single-core reference loop on the O projection (512-row slice scaled to 4096 rows): %.3f s"
                % (args.m, t_cpu, t_ref), "ms_per_step": round(t_cpu * 1e3, 2), "one_core_o_proj_s": round(t_ref, 3)}
+        # the reference's own host loop (skinny_gemm/test.cu:7-39, compiled from its source into oracle/_ref where
+        # the reference tree was present at build time), one core, same slice; it reads the bytes as E4M3 FNUZ
+        ref_lib = os.path.join(ROOT, "oracle", "_ref", "libref_host.so")
+        if os.path.exists(ref_lib):
+            import ctypes
+            import numpy as np
+            rl = ctypes.CDLL(ref_lib)
+            rl.ref_host_skinny_gemm_f32.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_float] + [ctypes.c_int] * 3
+            d = np.empty((args.m, 512), np.float32)
+            t0 = time.perf_counter()
+            rl.ref_host_skinny_gemm_f32(a8.ctypes.data, b8.ctypes.data, d.ctypes.data, 1.0, args.m, 512, k)
+            cpu["reference_host_loop_o_proj_s"] = round((time.perf_counter() - t0) * (n / 512.0), 3)
 
     out = {
         "metric": "achieved HBM TB/s (and us/GEMM), FP8 skinny GEMM, M=%d, Llama-3-8B projection shapes, 1 MI355X" % args.m,

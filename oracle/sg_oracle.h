@@ -14,6 +14,11 @@
  * The reference decodes E4M3 FNUZ through ROCm's hip_fp8.h and multiplies the two
  * operands as _Float16; this restatement decodes OCP E4M3 (the gfx950 MFMA
  * format) and multiplies in fp32, because 448*448 overflows fp16.
+ * orc_gemm_f32 and orc_tiled_sum_reduce are checked bit for bit against those two
+ * host loops themselves, compiled from the reference's sources (ref_host_loops.cpp ->
+ * _ref/libref_host.so, tests/test_reference_host.py): outside the three codes the
+ * formats read differently an FNUZ operand is exactly half the OCP one, so the
+ * reference's fp32 result is this library's times 1/4.
  *
  * Functions with no counterpart in the reference ("parity unpinned" by the
  * reference; pinned by closed forms, brute force and library casts in
