@@ -50,6 +50,23 @@ int launch_sparse(int mt, int rg, int xu2, int depth, const SparseArgs& sa, unsi
 // Prints a HIP failure to stderr when the environment variable SG_VERBOSE is set; returns e.
 hipError_t report_hip(const char* what, hipError_t e);
 
+// Dynamic LDS above the 48 KB default has to be requested per kernel and device.  `granted` (one array per
+// kernel, indexed by device) remembers the largest request already made, so that the launch path normally
+// makes no runtime call here; two threads racing on it at worst both make the same request.
+inline int request_dynamic_lds(const void* kernel, size_t lds, size_t (&granted)[16]) {
+    if (lds <= 48 * 1024) return SG_SUCCESS;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
+    if (granted[dev] >= lds) return SG_SUCCESS;
+    if (report_hip("hipFuncSetAttribute",
+                   hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
+        (void)hipGetLastError();
+        return SG_LAUNCH_FAILED;
+    }
+    granted[dev] = lds;
+    return SG_SUCCESS;
+}
+
 // Split-K workspace of the current device (created on first use).
 struct Workspace {
     float* partials = nullptr;

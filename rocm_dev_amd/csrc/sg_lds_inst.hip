@@ -18,22 +18,8 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
     else if constexpr (MODE == 3) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
     else if constexpr (MODE == 1) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false>;
     else kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
-    // dynamic LDS above the default cap must be requested per kernel; remember the largest
-    // request made so far on each device
-    static size_t attr_bytes[16] = {};
-    if (lds > 48 * 1024) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
-        if (attr_bytes[dev] < lds) {
-            if (report_hip("hipFuncSetAttribute",
-                           hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
-                (void)hipGetLastError();
-                return SG_LAUNCH_FAILED;
-            }
-            attr_bytes[dev] = lds;
-        }
-    }
+    static size_t granted[16] = {};
+    if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
     kernel<<<dim3(grid), dim3(threads), lds, stream>>>(a);
     return report_hip("lds_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }

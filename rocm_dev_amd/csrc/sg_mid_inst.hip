@@ -8,20 +8,8 @@ namespace sg {
 template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH>
 static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
     auto kernel = mid_gemm_kernel<RGW, MH, DEPTH, WN, DX>;
-    static size_t attr_bytes[16] = {};
-    if (lds > 48 * 1024) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
-        if (attr_bytes[dev] < lds) {
-            if (report_hip("hipFuncSetAttribute",
-                           hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
-                (void)hipGetLastError();
-                return SG_LAUNCH_FAILED;
-            }
-            attr_bytes[dev] = lds;
-        }
-    }
+    static size_t granted[16] = {};
+    if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
     kernel<<<dim3(grid), dim3(WN * 128), lds, stream>>>(a);
     return report_hip("mid_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }

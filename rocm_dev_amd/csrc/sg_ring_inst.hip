@@ -12,20 +12,8 @@ namespace sg {
 template <int BL, int XU>
 static int launch_one(int nt, const RingArgs& ra, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
     auto kernel = nt ? ring_gemm_kernel<SG_MT, BL, XU, true> : ring_gemm_kernel<SG_MT, BL, XU, false>;
-    static size_t attr_bytes[2][16] = {};
-    if (lds > 48 * 1024) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
-        if (attr_bytes[nt ? 1 : 0][dev] < lds) {
-            if (report_hip("hipFuncSetAttribute",
-                           hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
-                (void)hipGetLastError();
-                return SG_LAUNCH_FAILED;
-            }
-            attr_bytes[nt ? 1 : 0][dev] = lds;
-        }
-    }
+    static size_t granted[2][16] = {};
+    if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted[nt ? 1 : 0])) return rc;
     kernel<<<dim3(grid), dim3(threads), lds, stream>>>(ra);
     return report_hip("ring_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }

@@ -9,20 +9,8 @@ template <int MT, int RG, int XU2, int DEPTH>
 static int launch_one(const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
     if (threads > (unsigned)sparse_launch_bound(MT, RG)) return SG_INVALID_CONFIG;
     auto kernel = sparse24_gemm_kernel<MT, RG, XU2, DEPTH>;
-    static size_t attr_bytes[16] = {};
-    if (lds > 48 * 1024) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
-        if (attr_bytes[dev] < lds) {
-            if (report_hip("hipFuncSetAttribute",
-                           hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
-                (void)hipGetLastError();
-                return SG_LAUNCH_FAILED;
-            }
-            attr_bytes[dev] = lds;
-        }
-    }
+    static size_t granted[16] = {};
+    if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
     kernel<<<dim3(grid), dim3(threads), lds, stream>>>(sa);
     return report_hip("sparse24_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }
