@@ -110,7 +110,7 @@ struct Config {
 
 static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out) {
     const int frags = c.rg * c.mt;
-    if (c.waves < 1 || c.waves > 16 || c.depth < 1) return SG_INVALID_CONFIG;
+    if (c.waves < 1 || c.waves > 16 || c.depth < 1 || c.rg < 1 || c.mt < 1 || stage_bytes_k < 16) return SG_INVALID_CONFIG;
     a.waves = c.waves;
     a.split_k = c.split_k;
     a.n_tiles = (a.n + 16 * c.rg - 1) / (16 * c.rg);

@@ -465,6 +465,27 @@ def test_lds_ring_wave_tiles(sg, oracle, cfg, shape):
     assert np.array_equal(bits(D2), got)
 
 
+@pytest.mark.parametrize("field", ["waves", "row_tiles", "m_blocks", "depth", "k_chunks", "split_k"])
+@pytest.mark.parametrize("engine", [1, 2, 4])
+@pytest.mark.parametrize("bad", [0, -1, 1000])
+def test_tuning_record_with_a_nonsense_field_is_rejected(sg, engine, field, bad):
+    """A record from a stale or hand-edited tuning file must come back as an error code, not as a fault:
+    every field is checked before anything is launched."""
+    m, n, k = (64, 512, 1024) if engine == 4 else (8, 512, 1024)
+    A = torch.zeros((m, k), dtype=torch.uint8, device="cuda")
+    B = torch.zeros((n, k), dtype=torch.uint8, device="cuda")
+    D = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
+    kw = dict(engine=engine, split_k=1, waves=4, row_tiles=2, m_blocks=2 if engine == 4 else 1, depth=2,
+              k_chunks=4 if engine != 4 else 2)
+    kw[field] = bad
+    rc = sg.skinny_gemm_tuned(A, B, D, scale_tensor(1.0), **kw)
+    torch.cuda.synchronize()
+    if rc == 0:            # some values are legal for some engines (k_chunks of the LDS ring is ignored, ...)
+        assert torch.equal(D.float(), torch.zeros_like(D.float()))
+    else:
+        assert rc in (3, 4, 6, 10) and torch.equal(D.float(), torch.full_like(D.float(), 7.0))
+
+
 def test_torch_binding_surface(sg, oracle):
     """HFRK_skinny_gemm as the reference's Python callers use it: B passed as a (k, n) view."""
     m, n, k = 8, 1024, 2048
