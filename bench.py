@@ -134,9 +134,13 @@ def main():
             scl[(name, m)] = (sa * scales_b[name]).reshape(1).float().contiguous()
     torch.cuda.synchronize()
 
+    warm_cache = [False]     # True: every launch reads the same weight buffer (stays in the 256 MB last-level cache)
+
     def launch(name, m, i, stream):
         n, k = SHAPES[name]
         w = weights[name]
+        if warm_cache[0]:
+            i = 0
         rc = lib.sg_skinny_gemm_auto(acts[(name, m)].data_ptr(), w[i % len(w)].data_ptr(), outs[(name, m)].data_ptr(),
                                      scl[(name, m)].data_ptr(), m, n, k, k, stream)
         if rc != 0:
@@ -253,6 +257,12 @@ def main():
         nb = gemm_bytes(args.m, *SHAPES[name])
         per_shape[name] = {"us": round(b2b, 3), "TBps": round(nb / b2b / 1e6, 3), "frac_peak": round(nb / b2b / 1e6 / 8.0, 4),
                            "tuning": sg.skinny_gemm_pick(args.m, *SHAPES[name])}
+        # the same launches on ONE weight buffer: weights served by the last-level cache, not HBM - reported apart,
+        # never part of `value` or `roofline`
+        warm_cache[0] = True
+        warm = min(back_to_back_us(name, args.m, 60) for _ in range(3))
+        warm_cache[0] = False
+        per_shape[name]["warm_cache_us"] = round(warm, 3)
 
     sweep = None
     if not args.no_sweep:
