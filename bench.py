@@ -48,6 +48,7 @@ def main():
     ap.add_argument("--m", type=int, default=8, help="activation rows of the timed step")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-warm", action="store_true", help="skip the cache-resident (same weight buffer) timings")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs (for counter runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies (known traffic, to scale profiler counters)")
@@ -259,10 +260,11 @@ def main():
                            "tuning": sg.skinny_gemm_pick(args.m, *SHAPES[name])}
         # the same launches on ONE weight buffer: weights served by the last-level cache, not HBM - reported apart,
         # never part of `value` or `roofline`
-        warm_cache[0] = True
-        warm = min(back_to_back_us(name, args.m, 60) for _ in range(3))
-        warm_cache[0] = False
-        per_shape[name]["warm_cache_us"] = round(warm, 3)
+        if not args.no_warm:
+            warm_cache[0] = True
+            warm = min(back_to_back_us(name, args.m, 60) for _ in range(3))
+            warm_cache[0] = False
+            per_shape[name]["warm_cache_us"] = round(warm, 3)
 
     sweep = None
     if not args.no_sweep:
