@@ -94,3 +94,15 @@ def test_oracle_is_not_reachable_from_the_product():
             if f.endswith((".py", ".hip", ".h", ".cpp", "Makefile")):
                 text = open(os.path.join(dirpath, f), errors="ignore").read()
                 assert "liboracle" not in text and "import oracle" not in text and "sg_oracle" not in text, f
+
+
+def test_extension_module_name_and_signature():
+    """The reference's callers import `hfrk_skinny_gemm` and call one method with eleven arguments
+    (skinny_gemm/skinny_gemm_binding.cu:64-100)."""
+    import inspect
+
+    import hfrk_skinny_gemm
+    op = hfrk_skinny_gemm.HFRK_skinny_gemm(8)
+    params = list(inspect.signature(op.skinny_gemm_torch_binding).parameters)
+    assert params == ["A", "B", "D", "scale_tensor", "split_k", "A_producers", "B_producers", "consumers", "b_lanes",
+                      "qsize", "ops"]
