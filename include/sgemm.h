@@ -115,8 +115,9 @@ typedef struct SgTuning {
     int engine;        /* 0 library's choice, 1 direct (global -> VGPR -> MFMA), 2 LDS ring (global -> LDS DMA -> MFMA),
                           4 mid-batch (32 < m: weights streamed once, both operands staged in LDS for 2x2 or 4x2 waves) */
     int split_k;       /* workgroups sharing one output tile along K */
-    int waves;         /* wavefronts per workgroup, sharing the tile along K (1..16); mid-batch: 4 (2 along n x 2 along m)
-                          or 8 (4 x 2), each owning row_tiles x m_blocks fragments of the tile */
+    int waves;         /* wavefronts per workgroup, sharing the tile along K (1..16); mid-batch: 4 (2 along n x 2 along m),
+                          8 (4 x 2) or 14 (7 x 2, row_tiles = 2: 224-row tiles), each owning row_tiles x m_blocks
+                          fragments of the tile */
     int row_tiles;     /* 16-row weight tiles per wavefront (b_lanes); mid-batch: 2 or 4 */
     int m_blocks;      /* 16-row activation blocks per tile: 1 (m <= 16 per tile) or 2; mid-batch: 2, 4 or 8 per wavefront */
     int depth;         /* stages in flight per wavefront (register ring / LDS ring slots) */

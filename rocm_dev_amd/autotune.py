@@ -100,8 +100,10 @@ def search_space(m, n, k):
     authority: a candidate it has no kernel for comes back SG_INVALID_CONFIG and is skipped."""
     out = []
     if m > 32 and k % 128 == 0:
-        for waves, rt, mb, depth, dx, sk in itertools.product((4, 8), (2, 4), (2, 4, 8), (2, 3, 4, 6), (0, 2, 3), (1, 2, 4)):
+        for waves, rt, mb, depth, dx, sk in itertools.product((4, 8, 14), (2, 4), (2, 4, 8), (2, 3, 4, 6), (0, 2, 3), (1, 2, 4)):
             if dx and dx >= depth:
+                continue
+            if waves == 14 and rt != 2:             # 224-row tiles: seven waves along n, two fragments each
                 continue
             if 32 * mb >= 2 * m and mb > 2:      # tile more than twice as tall as the problem
                 continue

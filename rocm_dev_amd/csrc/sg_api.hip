@@ -265,10 +265,12 @@ static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
 static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) {
     if (a.k % 128 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if ((c.rg != 2 && c.rg != 4) || (c.mt != 2 && c.mt != 4 && c.mt != 8) || c.depth < 2) return SG_INVALID_CONFIG;
-    const int wn = c.waves == 8 ? 4 : 2;          // 8 waves = 4 (N) x 2 (M), otherwise 2 x 2
-    if (c.waves != 4 && c.waves != 8) return SG_INVALID_CONFIG;
+    if (c.waves != 4 && c.waves != 8 && c.waves != 14) return SG_INVALID_CONFIG;
+    const int wn = c.waves / 2;                   // waves = wn (along n) x 2 (along m)
     const int bn = 16 * c.rg * wn, bm = 32 * c.mt;
-    if (bn % (16 * wn) != 0 || bm % (16 * wn) != 0) return SG_INVALID_CONFIG;
+    // stage rows split evenly over the waves' 8-row DMA instructions (fourteen waves: the kernel gives the
+    // activation rows to the first eight)
+    if (bn % (16 * wn) != 0 || (wn != 7 && bm % (16 * wn) != 0)) return SG_INVALID_CONFIG;
     a.waves = c.waves;
     a.split_k = c.split_k;
     a.n_tiles = (a.n + bn - 1) / bn;
@@ -303,8 +305,10 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
 // long as every split keeps 32 K blocks.
 static Config pick_mid(int m, int n, int k, int cu_count) {
     struct Tile { int bn, bm, waves; };
+    // {224, 128, 14}: fourteen waves; 57344 = 256 x 224 gives every CU a tile where 256-row tiles fill 224 of 256
+    // (5 % at M = 128; at M = 256 the launch is power-bound and the fuller round gains nothing, so no 224 x 256)
     static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4},
-                                 {256, 128, 8}, {256, 64, 8}, {128, 256, 8}, {256, 256, 8}};
+                                 {256, 128, 8}, {224, 128, 14}, {256, 64, 8}, {128, 256, 8}, {256, 256, 8}};
     const int bm_max = m <= 64 ? 64 : (m <= 128 ? 128 : 256);
     const int blocks = k / 128;
     Config best;
@@ -316,6 +320,8 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
             if (sk > 1 && blocks / sk < 32) break;
             const long wgs = tiles * sk;
             const long rounds = (wgs + cu_count - 1) / cu_count;
+            // the fourteen-wave tile only where it is known to pay: unsplit, and exactly filling its rounds
+            if (t.waves == 14 && (sk > 1 || n % t.bn != 0 || wgs % cu_count != 0)) continue;
             const bool better = best_rounds < 0 || rounds < best_rounds ||
                                 (rounds == best_rounds && wgs * 16 > best_wgs * 17) ||   // clearly fuller round
                                 // as full with less splitting, when the splits had become short

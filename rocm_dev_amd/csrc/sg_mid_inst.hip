@@ -30,7 +30,16 @@ static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_
     if (rgw == RGW_ && mh == MH_ && depth == DEPTH_ && dx == DX_ && wn == 4)                   \
         return launch_one<RGW_, MH_, DEPTH_, 4, DX_>(a, grid, lds, stream);
 
+// fourteen-wave workgroups (7 along n x 2 along m): 224-row tiles
+#define SG_CASE_7(MH_, DEPTH_, DX_)                                                            \
+    if (rgw == 2 && mh == MH_ && depth == DEPTH_ && dx == DX_ && wn == 7)                      \
+        return launch_one<2, MH_, DEPTH_, 7, DX_>(a, grid, lds, stream);
+
 int launch_mid(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
+    SG_CASE_7(8, 3, 2) SG_CASE_7(8, 2, 2)                                       // 224 x 256: 84 + 64 KB
+    SG_CASE_7(4, 4, 2) SG_CASE_7(4, 4, 3) SG_CASE_7(4, 3, 3) SG_CASE_7(4, 3, 2)  // 224 x 128
+    SG_CASE_7(2, 4, 2) SG_CASE_7(2, 4, 4) SG_CASE_7(2, 3, 3)                     // 224 x 64
+    if (wn == 7) return SG_INVALID_CONFIG;
     SG_CASE(2, 2, 2) SG_CASE(2, 2, 3) SG_CASE(2, 2, 4) SG_CASE(2, 2, 6)
     SG_CASE(2, 4, 2) SG_CASE(2, 4, 3) SG_CASE(2, 4, 4) SG_CASE(2, 4, 6)
     SG_CASE(2, 8, 2) SG_CASE(2, 8, 3) SG_CASE(2, 8, 4)

@@ -33,12 +33,21 @@
 
 namespace sg {
 
-// RGW: 16-row weight fragments per wave (2 or 4)  -> BN = 32*RGW rows per workgroup
+// RGW: 16-row weight fragments per wave (2 or 4)  -> BN = 16*RGW*WN rows per workgroup
 // MH : 16-row activation fragments per wave (2, 4, 8) -> up to 32*MH activation rows per tile
-// WN : waves along N (2 or 4); the workgroup has WN x 2 waves
+// WN : waves along N (2, 4 or 7); the workgroup has WN x 2 waves.  WN = 7 makes 224-row tiles: 57344 = 256 x 224,
+//      one tile for each of the 256 CUs where 256-row tiles leave 32 CUs idle
 // DX : ring slots of the activations (<= DEPTH, the weights' ring slots).  The weights come from HBM,
 //      the activations from L2 with about half the latency; with DX < DEPTH the LDS a shallower
 //      activation ring frees buys the weights one more stage in flight.
+// waves that load the activation rows of a stage: the largest divisor of their `instr` DMA instructions <= waves
+constexpr int mid_activation_waves(int instr, int waves) {
+    int best = 1;
+    for (int d = 1; d <= waves; d++)
+        if (instr % d == 0) best = d;
+    return best;
+}
+
 template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH>
 __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) {
     // [DEPTH][W rows][128] | [DX][X rows][128], then (split-K only) 16 bytes for the arrival broadcast; no
@@ -48,9 +57,13 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     constexpr int WAVES = 2 * WN;
     constexpr int BN = 16 * RGW * WN;
     constexpr int BM = 32 * MH;
+    // The weight rows of a stage split evenly over all waves' DMA instructions (8 rows each); the activation rows
+    // over the first XW waves, XW = the largest divisor of their instruction count that is at most WAVES (all
+    // waves, except in fourteen-wave workgroups, where 32 or 16 or 8 instructions go to the first eight waves).
+    constexpr int XW = mid_activation_waves(BM / 8, WAVES);
     constexpr int W_INSTR = BN / 8 / WAVES;   // DMA instructions per wave per stage for the weights
-    constexpr int X_INSTR = BM / 8 / WAVES;   // ... and for the activations
-    static_assert(BN % (8 * WAVES) == 0 && BM % (8 * WAVES) == 0, "stage rows must split evenly over the waves' DMA instructions");
+    constexpr int X_INSTR = BM / 8 / XW;      // ... and for the activations, in the waves that load them
+    static_assert(BN % (8 * WAVES) == 0 && BM % (8 * XW) == 0, "stage rows must split evenly over the waves' DMA instructions");
     constexpr int PER_STAGE = W_INSTR + X_INSTR;
     constexpr int W_BYTES = BN * 128, X_BYTES = BM * 128;   // one ring slot of each operand
     constexpr int RING_BYTES = DEPTH * W_BYTES + DX * X_BYTES;
@@ -60,10 +73,13 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     constexpr int IN_FLIGHT_X = W_INSTR + (DX - 2) * PER_STAGE, IN_FLIGHT_W = (DEPTH - 2) * PER_STAGE;
     constexpr int IN_FLIGHT = IN_FLIGHT_X < IN_FLIGHT_W ? IN_FLIGHT_X : IN_FLIGHT_W;
     static_assert(IN_FLIGHT <= 63, "ring deeper than vmcnt can count");
+    // ... and in a wave that loads weights only, behind W(s) the weights of stages s+1 .. s+DEPTH-2:
+    constexpr int IN_FLIGHT_W_ONLY = (DEPTH - 2) * W_INSTR;
 
     const int lane = lane_id();
     const int wave = wave_id();
     const int wn = wave % WN, wm = wave / WN;
+    const bool loads_x = XW == WAVES || wave < XW;   // wave-uniform
 
     int bid = blockIdx.x;
     const int tile_n = bid % a.n_tiles;
@@ -93,7 +109,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     }
 #pragma unroll
     for (int i = 0; i < X_INSTR; i++) {
-        const int row_l = 8 * (WAVES * i + wave) + d_row;
+        const int row_l = 8 * (XW * i + (loads_x ? wave : 0)) + d_row;
         int row = m0 + row_l;
         row = row < a.m ? row : a.m - 1;
         xsrc[i] = a.A + (size_t)row * a.k + ((d_pp ^ ((row_l >> 1) & 7)) << 4);
@@ -102,9 +118,9 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     // DMA instruction i of a stage's refill: the activation instructions come first, then the weights'
     auto issue_one = [&](int i, int sx, int sw) __attribute__((always_inline)) {
         if (i < X_INSTR) {
-            if (sx < n_blk)
+            if (loads_x && sx < n_blk)
                 dma_1kb(xsrc[i] + ((size_t)(b_begin + sx) << 7),
-                        ring_lds + DEPTH * W_BYTES + (unsigned)(sx % DX) * X_BYTES + (WAVES * i + wave) * 1024);
+                        ring_lds + DEPTH * W_BYTES + (unsigned)(sx % DX) * X_BYTES + (XW * i + wave) * 1024);
         } else {
             if (sw < n_blk)
                 dma_1kb_stream(wsrc[i - X_INSTR] + ((size_t)(b_begin + sw) << 7),
@@ -212,8 +228,9 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     for (int s = 0; s < n_blk; s++) {
         // wait for this wave's part of stage s; everything issued after it may stay in flight.  Near the
         // end of the K range fewer stages follow, and the count is no longer known at compile time.
-        if (s + DEPTH - 2 < n_blk) wait_vmcnt<IN_FLIGHT>();
-        else wait_vmcnt<0>();
+        if (s + DEPTH - 2 >= n_blk) wait_vmcnt<0>();
+        else if (loads_x) wait_vmcnt<IN_FLIGHT>();
+        else wait_vmcnt<IN_FLIGHT_W_ONLY>();
         __syncthreads();        // stage s is complete for every wave; stage s-1 has been consumed by every wave
         __builtin_amdgcn_sched_barrier(0);
         // refills the slots of X(s-1) and W(s-1) on the way

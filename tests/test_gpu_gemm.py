@@ -370,6 +370,15 @@ MID_CONFIGS = [
     (2, 8, 4, 1, 8, 2),
     (2, 4, 6, 1, 8, 3),
     (2, 2, 4, 4, 8, 2),
+    # fourteen waves (7 x 2): 224-row tiles; the activation rows are loaded by the first eight waves
+    (2, 8, 3, 1, 14, 2),
+    (2, 8, 2, 1, 14),
+    (2, 8, 3, 4, 14, 2),
+    (2, 4, 4, 1, 14, 2),
+    (2, 4, 3, 2, 14),
+    (2, 4, 4, 1, 14, 3),
+    (2, 2, 4, 1, 14, 2),
+    (2, 2, 3, 4, 14),
 ]
 
 
