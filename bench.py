@@ -326,9 +326,11 @@ def main():
         mid = []
         for (n, k) in ((10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)):
             copies = max(2, int(COLD_BYTES // (n * k)) + 1)
-            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(copies)]
+            # N(0,1) operands quantised per tensor, as in the decode step (the code distribution matters: the
+            # MFMA-heavy shapes are power-limited, and uniformly random codes draw more power than real weights)
+            wb = [quantize(torch.randn((n, k), device="cuda", dtype=torch.float32))[0] for _ in range(copies)]
             for m in (64, 128, 256):
-                a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+                a8 = quantize(torch.randn((m, k), device="cuda", dtype=torch.float32))[0]
                 d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
                 one = torch.ones(1, device="cuda")
                 us = graph_time_us(lambda i, st: lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(),
@@ -339,14 +341,23 @@ def main():
         others["mid_batch"] = mid
         # 2:4 sparse GEMMs
         sp = []
-        nib = torch.tensor([0x4, 0x8, 0xC, 0x9, 0xD, 0xE], dtype=torch.uint8, device="cuda")
         for (n, k) in ((4096, 14336), (14336, 4096)):
             copies = max(2, int(COLD_BYTES // (n * k * 0.625)) + 1)
-            vb = [torch.randint(0, 0x7E, (n, k // 2), device="cuda", dtype=torch.uint8) for _ in range(copies)]
-            mb = [(nib[torch.randint(0, 6, (n, k // 8), device="cuda")] | (nib[torch.randint(0, 6, (n, k // 8), device="cuda")] << 4))
-                  for _ in range(copies)]
+            # N(0,1) weights quantised per tensor, then pruned 2:4 and compressed on the device
+            vb, mb = [], []
+            for _ in range(copies):
+                dense = quantize(torch.randn((n, k), device="cuda", dtype=torch.float32))[0]
+                v = torch.empty((n, k // 2), device="cuda", dtype=torch.uint8)
+                t = torch.empty((n, k // 8), device="cuda", dtype=torch.uint8)
+                rc = lib.sg_sparse24_compress(dense.data_ptr(), v.data_ptr(), t.data_ptr(), n, k, k, None)
+                if rc != 0:
+                    raise RuntimeError("sg_sparse24_compress: %s" % sg.strerror(rc))
+                vb.append(v)
+                mb.append(t)
+            torch.cuda.synchronize()
+            del dense
             for m in (1, 8, 16, 32):
-                a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+                a8 = quantize(torch.randn((m, k), device="cuda", dtype=torch.float32))[0]
                 d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
                 one = torch.ones(1, device="cuda")
                 us = graph_time_us(lambda i, st: lib.sg_sparse24_gemm(a8.data_ptr(), vb[i % copies].data_ptr(), mb[i % copies].data_ptr(),
