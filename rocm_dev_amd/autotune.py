@@ -121,12 +121,12 @@ def search_space(m, n, k):
             if lds_ring_fits(m, k, r):
                 out.append(r)
     for ku in (1, 2, 4, 8):
-        if k % (64 * ku):
-            continue
+        if ku > 1 and k % (64 * ku):
+            continue                              # (64-byte stages take any k: the last one may be partial)
         if k % 256 == 0 and ku != 4:
             continue                              # the LDS ring covers these; keep one direct family for comparison
         for sk, waves, rt, depth in itertools.product((1, 2, 4), (1, 2, 4, 8), (1, 2, 3, 4), (1, 2, 4)):
-            stages = k // (64 * ku)
+            stages = -(-k // (64 * ku))
             if sk * waves > stages:
                 continue
             out.append(record(ENGINE_DIRECT, sk, waves, rt, mb, depth, ku))

@@ -131,6 +131,10 @@ def test_search_space_respects_the_fit_rules():
     for (m, n, k) in [(8, 28672, 4096), (8, 4096, 4096), (32, 28672, 4096), (16, 4096, 14336)]:
         choice, _ = sg.skinny_gemm_choice(m, n, k)
         assert autotune_fields(choice) in autotune.search_space(m, n, k), (m, n, k, autotune_fields(choice))
+    # every k the library takes has candidates, down to a single partial 64-byte stage
+    for k in (16, 32, 48, 80, 4096 + 16):
+        space = autotune.search_space(8, 512, k)
+        assert space and all(r["engine"] == autotune.ENGINE_DIRECT and r["k_chunks"] == 1 for r in space), k
     # a k the LDS ring cannot take (not a multiple of 256) gets direct-engine candidates only
     assert {r["engine"] for r in autotune.search_space(8, 4096, 4096 + 64)} == {autotune.ENGINE_DIRECT}
     # mid-batch: the ring must fit 160 KB; 256 x 256 tiles only with a shallow activation ring
