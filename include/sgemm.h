@@ -203,8 +203,10 @@ int sg_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, 
 
 /* Per-row FP8 codec - no counterpart in the reference; the local compute on either side
  * of an FP8 all-reduce exchange.
- *   encode: scales[r] = absmax(X[r,:]) / 448 (1 if the row is all zero),
+ *   encode: scales[r] = absmax(X[r,:]) / 448 (1 if the row is all zero; NaNs do not count towards the maximum),
  *           Q[r,c] = e4m3_rne_sat( X[r,c] / scales[r] )                  (bit exact)
+ *           A NaN quotient (NaN input, or an infinite input in a row whose maximum is infinite) is 0x7f;
+ *           a finite input in such a row is a zero of its sign.
  *   decode: Y[r,c] = bf16( dec(Q[r,c]) * scales[r] )
  *   reduce: Y[r,c] = bf16( sum_{i<nbuf} dec(Q_i[r,c]) * scales_i[r] ), fp32, buffer order;
  *           buffer i starts at Q + i*q_buf_stride bytes, scales at scales + i*rows.

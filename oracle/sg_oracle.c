@@ -315,7 +315,11 @@ void orc_fp8_encode_rows(const uint16_t* X, uint8_t* Q, float* scales, int rows,
         for (int c = 0; c < cols; c++) { float a = fabsf(orc_bf16_to_f32(x[c])); if (a > amax) amax = a; }
         float s = (amax == 0.0f) ? 1.0f : amax / 448.0f;
         scales[r] = s;
-        for (int c = 0; c < cols; c++) Q[(size_t)r * cols + c] = orc_e4m3_encode(orc_bf16_to_f32(x[c]) / s);
+        for (int c = 0; c < cols; c++) {
+            /* a NaN quotient (NaN input, or inf / inf) is 0x7f whatever sign the division gave it */
+            const float q = orc_bf16_to_f32(x[c]) / s;
+            Q[(size_t)r * cols + c] = (q != q) ? 0x7f : orc_e4m3_encode(q);
+        }
     }
 }
 

@@ -95,7 +95,8 @@ void orc_gemm_sparse24_omp(const uint8_t* A, const uint8_t* vals, const uint8_t*
                            uint16_t* D, float scale, int m, int n, int k);
 
 /* ---- per-row FP8 codec (single-GPU half of an FP8 all-reduce) ----------- */
-/* X bf16 rows x cols; scale[r] = absmax(row)/448 (0 -> 1); Q = e4m3_rne_sat(x/scale) */
+/* X bf16 rows x cols; scale[r] = absmax(row)/448 (0 -> 1; NaNs ignored); Q = e4m3_rne_sat(x/scale),
+ * a NaN quotient (NaN input, inf/inf) -> 0x7f */
 void orc_fp8_encode_rows(const uint16_t* X, uint8_t* Q, float* scales, int rows, int cols);
 /* Y = bf16(dec(Q) * scale[r]) */
 void orc_fp8_decode_rows(const uint8_t* Q, const float* scales, uint16_t* Y, int rows, int cols);

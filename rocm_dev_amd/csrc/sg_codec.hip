@@ -30,6 +30,14 @@ __device__ __forceinline__ uint32_t cvt_bf16x2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, h);
 }
 
+// Both E4M3 NaN codes (0x7f, 0xff) -> 0x7f in all four bytes: the sign of a NaN quotient (NaN input, inf / inf)
+// depends on how the division is carried out, so the encoder's contract fixes it.
+__device__ __forceinline__ uint32_t canonical_nan_codes(int packed) {
+    const uint32_t u = (uint32_t)packed;
+    const uint32_t nan_sign = ((u & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u;   // bit 7 of every byte whose low seven bits are ones
+    return u & ~nan_sign;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
@@ -102,7 +110,7 @@ __global__ void __launch_bounds__(256) fp8_encode_rows_kernel(const uint16_t* __
         int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], 0, false);
         w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], w1, true);
         if (idx < nchunks) {
-            u32x2 out = {(uint32_t)w0, (uint32_t)w1};
+            u32x2 out = {canonical_nan_codes(w0), canonical_nan_codes(w1)};
             __builtin_nontemporal_store(out, qrow + idx);
         }
     }
@@ -144,7 +152,7 @@ __global__ void __launch_bounds__(256) fp8_encode_rows_long_kernel(const uint16_
         w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
         int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], 0, false);
         w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], w1, true);
-        qrow[idx] = u32x2{(uint32_t)w0, (uint32_t)w1};
+        qrow[idx] = u32x2{canonical_nan_codes(w0), canonical_nan_codes(w1)};
     }
 }
 

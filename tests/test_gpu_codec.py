@@ -132,3 +132,25 @@ def test_tiled_sum_reduce(sg, oracle, b, m, n):
     assert sg.tiled_sum_reduce(dev(A), dev(B), D) == 0
     torch.cuda.synchronize()
     assert np.array_equal(D.cpu().numpy(), oracle.tiled_sum_reduce(A, B))
+
+
+def test_encode_special_values_bit_exact(sg, oracle):
+    """Infinities, NaNs, denormals and signed zeros: same codes and scales as the oracle (whose values for these rows
+    are pinned in closed form by tests/test_oracle_gemm.py), and the decoder turns them back bit for bit."""
+    from test_oracle_gemm import _special_rows
+    X = np.tile(_special_rows(), (1, 300))
+    for cols in (64, 2560, 19200):                          # one wave, four waves with registers, the two-pass kernel
+        x = np.ascontiguousarray(X[:, :cols])
+        q_ref, s_ref = oracle.fp8_encode_rows(x)
+        Q = torch.empty(x.shape, dtype=torch.uint8, device="cuda")
+        S = torch.empty((x.shape[0],), dtype=torch.float32, device="cuda")
+        assert sg.fp8_encode_rows(dev(x), Q, S) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(Q.cpu().numpy(), q_ref)
+        assert np.array_equal(S.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
+        Y = torch.empty(x.shape, dtype=torch.bfloat16, device="cuda")
+        assert sg.fp8_decode_rows(Q, S, Y) == 0
+        torch.cuda.synchronize()
+        got, want = bits(Y), oracle.fp8_decode_rows(q_ref, s_ref)
+        nan = (want & 0x7FFF) > 0x7F80                       # NaN payloads are not part of the contract
+        assert np.array_equal(got[~nan], want[~nan]) and np.all((got[nan] & 0x7FFF) > 0x7F80)

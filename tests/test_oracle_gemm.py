@@ -299,3 +299,48 @@ def test_generator(oracle):
     cnt = int((np.abs(xf) == 50.0).sum())
     assert 0.99 * int(0.001 * n) <= cnt <= int(0.001 * n)
     assert (xf == 50.0).any() and (xf == -50.0).any()
+
+
+def _special_rows():
+    """Rows of non-finite and denormal bf16 inputs, with the codes and scale the encoder's contract gives them:
+    rows 0-2 are normal numbers with one +inf / -inf / NaN; 3-4 denormals; 5 all -0; 6 the largest finite value next
+    to the smallest normal; 7 +inf and NaN together; 8 all +inf; 9 all NaN; 10 all -inf but one +1.0."""
+    cols = 64
+    X = (np.arange(11 * cols, dtype=np.uint32).reshape(11, cols) * 37 % 0x100 + 0x3F00).astype(np.uint16)  # 0.5 .. 1 (bf16 bits)
+    X[:, ::2] |= 0x8000
+    X[0, 5], X[1, 7], X[2, 9] = 0x7F80, 0xFF80, 0x7FC0
+    X[3, :] = 0x0001
+    X[4, :] = 0x0000
+    X[4, 3] = 0x8001
+    X[5, :] = 0x8000
+    X[6, :] = 0x0000
+    X[6, 0], X[6, 1] = 0x7F7F, 0x0080
+    X[7, :] = 0x3F80
+    X[7, 2], X[7, 3] = 0x7FC0, 0x7F80
+    X[8, :] = 0x7F80
+    X[9, :] = 0xFFC0
+    X[10, :] = 0xFF80
+    X[10, 1] = 0x3F80
+    return X
+
+
+def test_encode_rows_special_values_closed_form(oracle):
+    X = _special_rows()
+    q, s = oracle.fp8_encode_rows(X)
+    sign = (X >> 8).astype(np.uint8) & 0x80
+    # an infinite maximum: scale inf; finite inputs become zeros of their sign, infinite ones (inf / inf) and NaNs 0x7f
+    for r in (0, 1, 7, 8, 10):
+        assert np.isinf(s[r]) and s[r] > 0
+        inf_or_nan = (X[r] & 0x7F80) == 0x7F80
+        assert np.array_equal(q[r][inf_or_nan], np.full(inf_or_nan.sum(), 0x7F, np.uint8))
+        assert np.array_equal(q[r][~inf_or_nan], sign[r][~inf_or_nan])
+    # a NaN does not enter the maximum: the row's scale is that of its finite values, its own code 0x7f
+    finite = oracle.bf16_to_f32(np.delete(X[2], 9))
+    assert s[2] == np.float32(np.abs(finite).max()) / np.float32(448.0) and q[2, 9] == 0x7F
+    assert np.array_equal(np.delete(q[2], 9), oracle.e4m3_encode(finite / s[2]))
+    # denormals: the maximum maps to 448 exactly like any other value
+    assert s[3] == np.float32(2.0 ** -133) / np.float32(448.0) and np.all(q[3] == 0x7E)
+    assert q[4, 3] == 0xFE and np.all(np.delete(q[4], 3) == 0)
+    assert s[5] == 1.0 and np.all(q[5] == 0x80)
+    assert q[6, 0] == 0x7E and q[6, 1] == 0 and np.all(q[6, 2:] == 0)
+    assert s[9] == 1.0 and np.all(q[9] == 0x7F)
