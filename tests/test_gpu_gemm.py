@@ -495,6 +495,27 @@ def test_tuning_record_with_a_nonsense_field_is_rejected(sg, engine, field, bad)
         assert rc in (3, 4, 6, 10) and torch.equal(D.float(), torch.full_like(D.float(), 7.0))
 
 
+@pytest.mark.parametrize("m,n,k", [(8, 512, 4096), (32, 1024, 1024), (5, 130, 272), (128, 1024, 2048), (256, 640, 4096),
+                                   (16, 28672, 4096)])
+def test_nan_codes_poison_exactly_their_row_and_column(sg, oracle, m, n, k):
+    """0x7f / 0xff are NaN in OCP E4M3 (and finite in the reference's FNUZ): an activation NaN poisons its output
+    row, a weight NaN its output column, nothing else - in every engine the shapes above reach."""
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=3)
+    a8[m // 2, k // 3] = 0x7F
+    b8[n // 2, k - 1] = 0xFF
+    b8[0, 0] = 0x7F
+    ref = oracle.gemm_omp(a8, b8, scale)
+    got = _run_fast(sg, a8, b8, scale)
+    nan_got, nan_ref = (got & 0x7FFF) > 0x7F80, (ref & 0x7FFF) > 0x7F80
+    want = np.zeros((m, n), bool)
+    want[m // 2, :] = True
+    want[:, n // 2] = True
+    want[:, 0] = True
+    assert np.array_equal(nan_ref, want) and np.array_equal(nan_got, want)
+    clean = lambda d, mask: np.where(mask, 0, d).astype(np.uint16)      # noqa: E731
+    assert oracle.max_rel_err_bf16(clean(got, want), clean(ref, want)) <= gemm_tol(k)
+
+
 def test_torch_binding_surface(sg, oracle):
     """HFRK_skinny_gemm as the reference's Python callers use it: B passed as a (k, n) view."""
     m, n, k = 8, 1024, 2048
