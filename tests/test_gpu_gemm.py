@@ -516,6 +516,48 @@ def test_nan_codes_poison_exactly_their_row_and_column(sg, oracle, m, n, k):
     assert oracle.max_rel_err_bf16(clean(got, want), clean(ref, want)) <= gemm_tol(k)
 
 
+def test_concurrent_launches_from_threads_on_their_own_streams(sg, oracle):
+    """The launchers keep no per-call state (skinny_gemm_caller.cu: enqueue on the given stream and return), so host
+    threads may launch at the same time on different streams; split-K shapes are left out because their workspace is
+    one per device.  Every thread's results must equal the ones computed alone, bit for bit."""
+    import threading
+    shapes = [(8, 4096, 4096), (32, 6144, 1024), (128, 1024, 2048), (16, 2000, 528)]
+    work = []
+    for i, (m, n, k) in enumerate(shapes):
+        a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=30 + i)
+        A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+        alone = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
+        assert sg.skinny_gemm_fastpath(A, B, alone, S) == 0
+        work.append((A, B, S, alone))
+    torch.cuda.synchronize()
+    errors = []
+
+    def run(idx):
+        try:
+            A, B, S, alone = work[idx]
+            stream = torch.cuda.Stream()
+            outs = [torch.full_like(alone, float("nan")) for _ in range(4)]
+            with torch.cuda.stream(stream):
+                for rep in range(40):
+                    rc = sg.skinny_gemm_fastpath(A, B, outs[rep % 4], S)
+                    if rc != 0:
+                        errors.append((idx, rc))
+                        return
+            stream.synchronize()
+            for o in outs:
+                if not torch.equal(o.view(torch.int16), alone.view(torch.int16)):
+                    errors.append((idx, "result differs"))
+        except Exception as e:      # surface it in the main thread
+            errors.append((idx, repr(e)))
+
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(len(shapes)) for _ in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 def test_torch_binding_surface(sg, oracle):
     """HFRK_skinny_gemm as the reference's Python callers use it: B passed as a (k, n) view."""
     m, n, k = 8, 1024, 2048
