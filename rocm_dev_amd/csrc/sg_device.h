@@ -10,6 +10,7 @@ namespace sg {
 typedef long  i64x2 __attribute__((ext_vector_type(2)));
 typedef int   i32x2 __attribute__((ext_vector_type(2)));
 typedef int   i32x4 __attribute__((ext_vector_type(4)));
+typedef int   i32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
@@ -38,6 +39,15 @@ __device__ __forceinline__ i64x2 load16(const void* p) { return *reinterpret_cas
 __device__ __forceinline__ i64x2 load16_stream(const void* p) {
     return __builtin_nontemporal_load(reinterpret_cast<const i64x2*>(p));
 }
+
+// D = A x B + C on gfx950's FP8 matrix core: 16 x 16 outputs, 128 bytes of K per instruction, both operands OCP E4M3
+// (format codes 0/0).  The builtin is the block-scaled form; with both scale operands the constant 0 the compiler
+// emits the plain v_mfma_f32_16x16x128_f8f6f4 - no scale-load instruction in front of every MFMA, bit-identical
+// results to unit scales (E8M0 byte 127), and about 7 % more sustained throughput on real data (less power).
+__device__ __forceinline__ f32x4 mfma_e4m3_16x16x128(const i32x8& a, const i32x8& b, const f32x4& c) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+
 
 // Workgroups are dispatched round-robin over the 8 XCDs (workgroup b runs on XCD b % 8), each with its own
 // L2.  A 16-row tile writes only 32 bytes of every output row, so the four tiles that share a 128-byte line of

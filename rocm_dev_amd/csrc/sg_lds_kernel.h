@@ -73,11 +73,10 @@ __device__ __forceinline__ void drain_ring(Consume& consume, int i) {
     if constexpr (D + 1 < DEPTH) drain_ring<D + 1, DEPTH, PER_STAGE>(consume, i);
 }
 
-typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 // One 256-byte K block of a stage: weights at w (16*RG rows, 4 KB per 16-row tile), activations
 // at x (4 KB per 16-row block), both already offset by the lane's read offset.  The four 64-byte
-// chunks of the block feed two v_mfma_scale_f32_16x16x128_f8f6f4 (unit scales): lane (r, g)
+// chunks of the block feed two v_mfma_f32_16x16x128_f8f6f4: lane (r, g)
 // supplies its 16-byte pieces of chunks 0,1 to the first and of chunks 2,3 to the second - the
 // same pieces for both operands, so the K permutation cancels.  The 128-wide instruction runs at
 // the full FP8 rate of gfx950 (measured 4.9 PFLOP/s against 0.8-1.3 for v_mfma_f32_16x16x32_fp8_fp8).
@@ -101,8 +100,7 @@ __device__ __forceinline__ void mma_block_256(const uint8_t* w, const uint8_t* x
             const i32x8 wv = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
-                acc[rg][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, xv[mt][h], acc[rg][mt], 0, 0, 0, 0x7f7f7f7f, 0,
-                                                                               0x7f7f7f7f);
+                acc[rg][mt] = mfma_e4m3_16x16x128(wv, xv[mt][h], acc[rg][mt]);
         }
 }
 

@@ -8,8 +8,8 @@
 // Waves form a 2 x 2 grid over the tile: wave (wn, wm) owns 16*RGW weight rows and 16*MH
 // activation rows, so each weight fragment it reads from LDS feeds MH MFMAs and each
 // activation fragment RGW MFMAs - the register-level reuse that keeps LDS bandwidth (128
-// B/clk/CU) under the MFMA rate.  The MFMA is gfx950's v_mfma_scale_f32_16x16x128_f8f6f4
-// with unit block scales: 128 bytes of K per instruction, i.e. one instruction per stage and
+// B/clk/CU) under the MFMA rate.  The MFMA is gfx950's v_mfma_f32_16x16x128_f8f6f4
+// (no block scales): 128 bytes of K per instruction, i.e. one instruction per stage and
 // fragment pair.  Lane (r = l%16, g = l/16) supplies 32 bytes of row r; which 32 bytes is
 // free as long as both operands agree, so both take 16-byte pieces g and g+4 of the block.
 //
@@ -180,9 +180,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int rg = 0; rg < RGW; rg++)
-                // formats 0/0 = OCP E4M3 for both operands; E8M0 scale byte 127 = 2^0 for both
-                acc[rg][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w[rg], x[mb & 1], acc[rg][mb], 0, 0, 0,
-                                                                               0x7f7f7f7f, 0, 0x7f7f7f7f);
+                acc[rg][mb] = mfma_e4m3_16x16x128(w[rg], x[mb & 1], acc[rg][mb]);
             // an MFMA has no side effects and its result is not read before the next stage, so the
             // optimizer would sink the group behind the reads and (conditional) refills that follow, and
             // hoist every read to the top; naming the accumulators as operands of an asm with a memory
@@ -215,8 +213,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
             const i32x8 w = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
             for (int mb = 0; mb < MH; mb++)
-                acc[rg][mb] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, x[mb], acc[rg][mb], 0, 0, 0, 0x7f7f7f7f,
-                                                                               0, 0x7f7f7f7f);
+                acc[rg][mb] = mfma_e4m3_16x16x128(w, x[mb], acc[rg][mb]);
         }
     };
 

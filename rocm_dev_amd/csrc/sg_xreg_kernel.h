@@ -97,8 +97,7 @@ __global__ void __launch_bounds__(xreg_launch_bound(MT, RG, PT)) lds_gemm_xreg_k
                 const i32x8 wv = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++)
-                    acc[rg][mt] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wv, x[mt][h], acc[rg][mt], 0, 0, 0, 0x7f7f7f7f,
-                                                                                   0, 0x7f7f7f7f);
+                    acc[rg][mt] = mfma_e4m3_16x16x128(wv, x[mt][h], acc[rg][mt]);
             }
     };
 
