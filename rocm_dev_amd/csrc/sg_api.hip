@@ -305,10 +305,10 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
 // long as every split keeps 32 K blocks.
 static Config pick_mid(int m, int n, int k, int cu_count) {
     struct Tile { int bn, bm, waves; };
-    // {224, 128, 14}: fourteen waves; 57344 = 256 x 224 gives every CU a tile where 256-row tiles fill 224 of 256
-    // (5 % at M = 128; at M = 256 the launch is power-bound and the fuller round gains nothing, so no 224 x 256)
-    static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4},
-                                 {256, 128, 8}, {224, 128, 14}, {256, 64, 8}, {128, 256, 8}, {256, 256, 8}};
+    // {224, *, 14}: fourteen waves; 57344 = 256 x 224 gives every CU a tile where 256-row tiles fill 224 of 256
+    // (5-10 % at M = 128 and 256 on N(0,1)-quantised operands)
+    static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4}, {256, 128, 8}, {224, 128, 14},
+                                 {256, 64, 8}, {128, 256, 8}, {256, 256, 8}, {224, 256, 14}};
     const int bm_max = m <= 64 ? 64 : (m <= 128 ? 128 : 256);
     const int blocks = k / 128;
     Config best;
@@ -320,8 +320,9 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
             if (sk > 1 && blocks / sk < 32) break;
             const long wgs = tiles * sk;
             const long rounds = (wgs + cu_count - 1) / cu_count;
-            // the fourteen-wave tile only where it is known to pay: unsplit, and exactly filling its rounds
-            if (t.waves == 14 && (sk > 1 || n % t.bn != 0 || wgs % cu_count != 0)) continue;
+            // the fourteen-wave tile only where it is known to pay: unsplit, one tile covering all of m (the
+            // weights streamed once), and exactly filling its rounds
+            if (t.waves == 14 && (sk > 1 || m > t.bm || n % t.bn != 0 || wgs % cu_count != 0)) continue;
             const bool better = best_rounds < 0 || rounds < best_rounds ||
                                 (rounds == best_rounds && wgs * 16 > best_wgs * 17) ||   // clearly fuller round
                                 // as full with less splitting, when the splits had become short
