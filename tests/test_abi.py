@@ -106,3 +106,29 @@ def test_extension_module_name_and_signature():
     params = list(inspect.signature(op.skinny_gemm_torch_binding).parameters)
     assert params == ["A", "B", "D", "scale_tensor", "split_k", "A_producers", "B_producers", "consumers", "b_lanes",
                       "qsize", "ops"]
+
+
+def test_compat_header_compiles_against_a_reference_style_main(tmp_path):
+    """include/sgemm_compat.hpp: a main written like the reference's test.cu (calls by the original names) compiles
+    and links against libsgemm.so; it is not run here (no device)."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    src = tmp_path / "main.cpp"
+    src.write_text("""
+#include "sgemm_compat.hpp"
+int main() {
+    fp8 *A = nullptr, *B = nullptr; unsigned short* D = nullptr; float *S = nullptr, *F = nullptr;
+    int rc = skinny_gemm_fastpath(A, B, D, S, 8, 4096, 4096);
+    rc += skinny_gemm(A, B, D, S, 8, 4096, 4096, 4096, 1, 0, 0, 4, 1, 2, 16, 4, (hipStream_t)0);
+    rc += async_gemm<float>(A, B, F, 8, 64, 256) + async_gemm<unsigned short>(A, B, D, 8, 64, 256);
+    rc += tiled_sum_reduce(F, F, F, 2, 8, 64);
+    return rc == 0;
+}
+""")
+    lib_dir = os.path.join(ROOT, "rocm_dev_amd", "csrc")
+    out = tmp_path / "main.out"
+    res = subprocess.run([hipcc, "-x", "hip", "--cuda-host-only", "-O1", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(out),
+                          "-L", lib_dir, "-lsgemm", "-Wl,-rpath," + lib_dir], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert out.exists()
