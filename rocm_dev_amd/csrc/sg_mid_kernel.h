@@ -25,6 +25,8 @@
 //
 // K is split across workgroups when there are few tiles; partials meet in the fp32 workspace
 // and the last workgroup to arrive sums them in split order (same scheme as the skinny path).
+// Inside its K range a workgroup starts at a block that depends on its weight tile and wraps
+// around, so the fp32 sum of an output element is taken in a rotated - still fixed - K order.
 #pragma once
 
 #include "sg_device.h"
@@ -94,6 +96,15 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     const int b_begin = split * per_split;
     const int b_end = (split == a.split_k - 1) ? blocks : b_begin + per_split;
     const int n_blk = b_end - b_begin;
+    // Every workgroup walks its K range from a different starting block (and wraps): workgroups that start
+    // together would otherwise ask one L2 for the same activation lines at the same moment, block after
+    // block, and queue up at one channel.  The start depends on the weight tile only, so the workgroups that
+    // share weight rows (other activation tiles) still read them together and HBM serves them once.
+    const int k_rot = (int)((((unsigned)tile_n >> 3) * 5u) % (unsigned)n_blk);
+    auto k_block = [&](int s) __attribute__((always_inline)) {
+        const int b = s + k_rot;
+        return b_begin + (b >= n_blk ? b - n_blk : b);
+    };
 
     // ---- DMA sources: instruction i of this wave covers stage rows 8*(4*i + wave) .. +7 ------
     const int d_row = lane >> 3;                 // row inside the 8-row instruction
@@ -119,11 +130,11 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     auto issue_one = [&](int i, int sx, int sw) __attribute__((always_inline)) {
         if (i < X_INSTR) {
             if (loads_x && sx < n_blk)
-                dma_1kb(xsrc[i] + ((size_t)(b_begin + sx) << 7),
+                dma_1kb(xsrc[i] + ((size_t)k_block(sx) << 7),
                         ring_lds + DEPTH * W_BYTES + (unsigned)(sx % DX) * X_BYTES + (XW * i + wave) * 1024);
         } else {
             if (sw < n_blk)
-                dma_1kb_stream(wsrc[i - X_INSTR] + ((size_t)(b_begin + sw) << 7),
+                dma_1kb_stream(wsrc[i - X_INSTR] + ((size_t)k_block(sw) << 7),
                                ring_lds + (unsigned)(sw % DEPTH) * W_BYTES + (WAVES * (i - X_INSTR) + wave) * 1024);
         }
     };
