@@ -470,9 +470,13 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     const unsigned my_ring_lds = lds_addr(my_ring);
     const unsigned x_lds = lds_addr(ring);
 
-    // ---- resident activations: K block kb is fetched by wave kb % waves (m_tiles == 1) ----------
+    // ---- resident activations (m_tiles == 1): the waves share out the K blocks, starting at a block that differs
+    // from workgroup to workgroup - all workgroups fetch the same lines from L2 at launch, and in the same order
+    // they would all be at the same channel at the same time (4 % of the launch at m = 32)
     int x_issued = 0;
-    for (int kb = wave; kb < blocks; kb += waves) {
+    const int x_rot = (int)(((unsigned)blockIdx.x * 3u) % (unsigned)blocks);
+    for (int kb0 = wave; kb0 < blocks; kb0 += waves) {
+        const int kb = kb0 + x_rot >= blocks ? kb0 + x_rot - blocks : kb0 + x_rot;
 #pragma unroll
         for (int u = 0; u < XU; u++) {
             int row = 4 * u + src_row;
