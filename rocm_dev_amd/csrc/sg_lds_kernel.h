@@ -456,9 +456,11 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     const int gw = (int)blockIdx.x * waves + wave;
     const int my_tiles = gw < total_tiles ? (total_tiles - gw + total_waves - 1) / total_waves : 0;
     const int total = blocks * my_tiles;
-    // Every wave starts its tiles at a different K block and wraps around.  Waves that all ask for block kb of
-    // their rows at the same moment load the memory channels unevenly (row pitches are multiples of 4 KB);
-    // spread over all K offsets the same stream runs about 4 % faster (measured on 8 x 28672 x 4096).
+    // Every wave starts its tiles at a different K block and wraps around.  Here all waves of the chip would
+    // otherwise ask for block kb of their rows at the same moment, and row pitches are multiples of 4 KB: in step,
+    // 8 x 28672 x 4096 takes 24.6 us, spread over all K offsets 19.6 us (eight waves, same process, interleaved).
+    // The persistent K-split kernel above already has its waves at different K offsets and measured 1 % slower
+    // with a shift per workgroup on top; it keeps plain K order.
     const int k_rot = (int)((unsigned)gw % (unsigned)blocks);
 
     const int q = lane >> 2, p = lane & 3;
@@ -470,13 +472,9 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     const unsigned my_ring_lds = lds_addr(my_ring);
     const unsigned x_lds = lds_addr(ring);
 
-    // ---- resident activations (m_tiles == 1): the waves share out the K blocks, starting at a block that differs
-    // from workgroup to workgroup - all workgroups fetch the same lines from L2 at launch, and in the same order
-    // they would all be at the same channel at the same time (4 % of the launch at m = 32)
+    // ---- resident activations: K block kb is fetched by wave kb % waves (m_tiles == 1) ----------
     int x_issued = 0;
-    const int x_rot = (int)(((unsigned)blockIdx.x * 3u) % (unsigned)blocks);
-    for (int kb0 = wave; kb0 < blocks; kb0 += waves) {
-        const int kb = kb0 + x_rot >= blocks ? kb0 + x_rot - blocks : kb0 + x_rot;
+    for (int kb = wave; kb < blocks; kb += waves) {
 #pragma unroll
         for (int u = 0; u < XU; u++) {
             int row = 4 * u + src_row;

@@ -52,6 +52,15 @@ __global__ void __launch_bounds__(xreg_launch_bound(MT, RG, PT)) lds_gemm_xreg_k
     const TileRun run = persistent_tile_run(total_tiles);
     const int my_tiles = run.count;
     const int total = streaming ? PT * my_tiles : 0;             // stages of this wave
+    // wave w works on K blocks w, w + waves, ... shifted by an amount that differs from workgroup to workgroup
+    // (and wrapped), so that the workgroups of the chip are spread over all K offsets at any moment
+    // (1 % on 32 x 28672 x 4096, interleaved same-process runs)
+    const int blocks = PT * waves;
+    const int k_rot = (int)(((unsigned)blockIdx.x * 3u) % (unsigned)blocks);
+    auto k_block = [&](int t) __attribute__((always_inline)) {
+        const int kb = wave + t * waves + k_rot;
+        return kb >= blocks ? kb - blocks : kb;
+    };
 
     // ---- weight ring ------------------------------------------------------------------------------
     const int q = lane >> 2, p = lane & 3;
@@ -62,11 +71,11 @@ __global__ void __launch_bounds__(xreg_launch_bound(MT, RG, PT)) lds_gemm_xreg_k
     const unsigned my_ring_lds = lds_addr(my_ring);
     f32x4* red = reinterpret_cast<f32x4*>(ring + (size_t)waves * (DEPTH * STAGE_BYTES));
 
-    auto issue = [&](int i) __attribute__((always_inline)) {   // stage i = tile i / PT, K block wave + (i % PT) * waves
+    auto issue = [&](int i) __attribute__((always_inline)) {   // stage i = tile i / PT, K block k_block(i % PT)
         const int j = i / PT, t = i % PT;
         const int n0 = (run.first + j) * (16 * RG);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
-        const size_t koff = ((size_t)(wave + t * waves) << 8) + src_col;
+        const size_t koff = ((size_t)k_block(t) << 8) + src_col;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
 #pragma unroll
@@ -152,7 +161,7 @@ __global__ void __launch_bounds__(xreg_launch_bound(MT, RG, PT)) lds_gemm_xreg_k
         for (int mt = 0; mt < MT; mt++) {
             int row = mt * 16 + r;
             row = row < a.m ? row : a.m - 1;   // rows past the edge repeat the last one; never stored
-            const uint8_t* src = a.A + (size_t)row * a.k + ((size_t)(wave + t * waves) << 8) + 16 * g;
+            const uint8_t* src = a.A + (size_t)row * a.k + ((size_t)k_block(t) << 8) + 16 * g;
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 const i32x4 lo = __builtin_bit_cast(i32x4, load16(src + (2 * h) * 64));
