@@ -306,9 +306,9 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
 static Config pick_mid(int m, int n, int k, int cu_count) {
     struct Tile { int bn, bm, waves; };
     // {224, *, 14}: fourteen waves; 57344 = 256 x 224 gives every CU a tile where 256-row tiles fill 224 of 256
-    // (5-10 % at M = 128 and 256 on N(0,1)-quantised operands)
+    // (5-10 % at M = 128 and 256 on N(0,1)-quantised operands, 4 % at M = 64 over two co-resident 128 x 64 tiles)
     static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4}, {256, 128, 8}, {224, 128, 14},
-                                 {256, 64, 8}, {128, 256, 8}, {256, 256, 8}, {224, 256, 14}};
+                                 {256, 64, 8}, {224, 64, 14}, {128, 256, 8}, {256, 256, 8}, {224, 256, 14}};
     const int bm_max = m <= 64 ? 64 : (m <= 128 ? 128 : 256);
     const int blocks = k / 128;
     Config best;
@@ -339,7 +339,7 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     }
     Config c = best;
     bool co_resident = false;
-    if (m <= 64 && (long)((n + 127) / 128) * 2 >= 3L * cu_count) {
+    if (m <= 64 && c.waves != 14 && (long)((n + 127) / 128) * 2 >= 3L * cu_count) {
         // memory-bound and many tiles: several small two-slot workgroups per CU hide the DMA
         // latency better than one deep ring
         c.waves = 8; c.rg = 2; c.mt = 2; c.split_k = 1;
@@ -353,8 +353,8 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     const int per_wave_w = bn / (8 * c.waves), per_wave_x = bm / (8 * c.waves);   // DMA instructions per wave and stage
     // (weight slots, activation slots; 0 = as many): the deepest ring that fits 160 KB.  A shallower
     // activation ring (activations come from L2, weights from HBM) is what lets the 256 x 256 tile keep
-    // two weight stages in flight.
-    static const int rings[][2] = {{4, 0}, {3, 0}, {3, 2}, {2, 0}};
+    // two weight stages in flight, and the 224 x 128 tile three (86 -> 80 us at 128 x 57344 x 8192).
+    static const int rings[][2] = {{4, 0}, {4, 3}, {3, 0}, {3, 2}, {2, 0}};
     c.depth = 2;
     c.ku = 0;
     if (co_resident) {
@@ -363,6 +363,7 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     } else {
         for (const auto& r : rings) {
             const int dw = r[0], dx = r[1] ? r[1] : r[0];
+            if (dw == 4 && dx == 3 && c.waves != 14) continue;   // compiled for the 224 x 128 tile, which it fills to 160 KB
             const int in_flight_x = per_wave_w + (dx - 2) * (per_wave_w + per_wave_x);
             const int in_flight_w = (dw - 2) * (per_wave_w + per_wave_x);
             const size_t lds = ((size_t)dw * bn + (size_t)dx * bm) * 128 + (c.split_k > 1 ? 16 : 0);   // + arrival word

@@ -5,7 +5,7 @@ import ctypes as C
 
 import pytest
 
-from rocm_dev_amd import autotune
+from rocm_dev_amd import api, autotune
 
 
 @pytest.fixture()
@@ -145,3 +145,30 @@ def test_search_space_respects_the_fit_rules():
     for shape in [(256, 57344, 8192), (128, 8192, 8192), (64, 8192, 28672), (64, 10240, 8192)]:
         choice, _ = sg.skinny_gemm_choice(*shape)
         assert autotune_fields(choice) in autotune.search_space(*shape), shape
+
+
+def test_same_launch_reads_mid_batch_activation_slots_like_the_library():
+    """k_chunks = 0 (or anything outside 2 .. depth - 1) means "as many activation slots as weight slots" to the
+    mid-batch engine, so such records are one launch; any other field that differs makes two."""
+    mid = autotune.record(autotune.ENGINE_MID, 1, 14, 2, 2, 4, 0)
+    assert autotune.same_launch(mid, dict(mid, k_chunks=4))
+    assert autotune.same_launch(mid, dict(mid, k_chunks=7))
+    assert not autotune.same_launch(mid, dict(mid, k_chunks=3))
+    assert not autotune.same_launch(mid, dict(mid, depth=3))
+    lds = autotune.record(autotune.ENGINE_LDS, 1, 8, 1, 1, 2, 4, 1, 1, 6)
+    assert autotune.same_launch(lds, dict(lds))
+    assert not autotune.same_launch(lds, dict(lds, k_chunks=0))
+
+
+def test_heuristics_pick_the_fourteen_wave_tile_where_it_fills_the_chip():
+    """57344 = 256 x 224: one 224-row tile per CU for every m the tile covers, three weight slots in flight where the
+    tile leaves room (224 x 128: 4 + 3 slots are exactly 160 KB)."""
+    for m, mb, depth, dx in ((48, 2, 4, 4), (64, 2, 4, 4), (128, 4, 4, 3), (256, 8, 3, 2)):
+        t, from_table = api.skinny_gemm_choice(m, 57344, 8192)
+        assert not from_table
+        got = (t.engine, t.split_k, t.waves, t.row_tiles, t.m_blocks, t.depth, t.k_chunks if t.k_chunks else t.depth)
+        assert got == (autotune.ENGINE_MID, 1, 14, 2, mb, depth, dx), (m, got)
+    # a row count that 224 does not divide, or more rows than one tile covers: eight-wave tiles as before
+    for m, n in ((64, 57344 + 128), (300, 57344)):
+        t, _ = api.skinny_gemm_choice(m, n, 8192)
+        assert t.waves != 14, (m, n)
