@@ -284,7 +284,8 @@ def main(argv=None):
     ap.add_argument("--top", type=int, default=1, help="print this many best candidates per shape")
     ap.add_argument("--launches", type=int, default=20, help="launches per timed graph")
     ap.add_argument("--min-gain", type=float, default=0.02,
-                    help="keep a shape out of the table unless the winner beats the built-in choice by this fraction")
+                    help="keep a shape out of the table unless the winner beats the built-in choice by this fraction "
+                         "(negative: always record the winner, even the built-in choice itself)")
     ap.add_argument("--limit", type=int, default=None, help="time only the first N candidates (smoke runs)")
     args = ap.parse_args(argv)
     shapes = [tuple(int(x) for x in s.lower().split("x")) for s in args.shapes]
@@ -302,7 +303,7 @@ def main(argv=None):
         from .api import skinny_gemm_choice
         own, _ = skinny_gemm_choice(m, n, k)
         own = {f: getattr(own, f) for f in FIELDS}
-        if kept and kept[0][0] < base_us * (1.0 - args.min_gain) and not same_launch(kept[0][1], own):
+        if kept and kept[0][0] < base_us * (1.0 - args.min_gain) and (args.min_gain < 0 or not same_launch(kept[0][1], own)):
             entries[(m, n, k)] = kept[0][1]
         else:
             entries.pop((m, n, k), None)
