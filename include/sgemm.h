@@ -15,7 +15,10 @@
  *   - D is OVERWRITTEN (the reference accumulates with atomics into a pre-zeroed D);
  *   - D is bf16 (the reference writes fp16 or fp32);
  *   - split-K partial sums are reduced in fp32 in a fixed order, so results are
- *     bit-reproducible from run to run.
+ *     bit-reproducible from run to run.  The order in which one output element's K
+ *     products are summed is a property of the configuration that runs (which waves
+ *     and workgroups share K, and at which K block each of them starts); two
+ *     configurations may differ in the last bit of the fp32 sum before rounding.
  *
  * Reference citations are paths below the reference tree's projects/ directory.
  */
