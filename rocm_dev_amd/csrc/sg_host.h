@@ -5,6 +5,9 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <mutex>
+
 #include "../../include/sgemm.h"
 
 namespace sg {
@@ -51,19 +54,24 @@ int launch_sparse(int mt, int rg, int xu2, int depth, const SparseArgs& sa, unsi
 hipError_t report_hip(const char* what, hipError_t e);
 
 // Dynamic LDS above the 48 KB default has to be requested per kernel and device.  `granted` (one array per
-// kernel, indexed by device) remembers the largest request already made, so that the launch path normally
-// makes no runtime call here; two threads racing on it at worst both make the same request.
-inline int request_dynamic_lds(const void* kernel, size_t lds, size_t (&granted)[16]) {
+// kernel, indexed by device, zero-initialised static storage) remembers the largest request already made, so
+// that the launch path normally makes no runtime call here.  Raising the limit is serialised: a smaller request
+// that overtook a larger one would otherwise lower the attribute under the larger one's launch.
+typedef std::atomic<size_t> LdsGranted[16];
+inline int request_dynamic_lds(const void* kernel, size_t lds, LdsGranted& granted) {
     if (lds <= 48 * 1024) return SG_SUCCESS;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return SG_NO_DEVICE;
-    if (granted[dev] >= lds) return SG_SUCCESS;
+    if (granted[dev].load(std::memory_order_acquire) >= lds) return SG_SUCCESS;
+    static std::mutex raise;
+    std::lock_guard<std::mutex> lock(raise);
+    if (granted[dev].load(std::memory_order_relaxed) >= lds) return SG_SUCCESS;
     if (report_hip("hipFuncSetAttribute",
                    hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)) != hipSuccess) {
         (void)hipGetLastError();
         return SG_LAUNCH_FAILED;
     }
-    granted[dev] = lds;
+    granted[dev].store(lds, std::memory_order_release);
     return SG_SUCCESS;
 }
 

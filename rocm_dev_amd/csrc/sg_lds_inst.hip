@@ -18,7 +18,7 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
     else if constexpr (MODE == 3) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
     else if constexpr (MODE == 1) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false>;
     else kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
-    static size_t granted[16] = {};
+    static LdsGranted granted;
     if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
     kernel<<<dim3(grid), dim3(threads), lds, stream>>>(a);
     return report_hip("lds_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;

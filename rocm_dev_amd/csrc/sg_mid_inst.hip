@@ -8,7 +8,7 @@ namespace sg {
 template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH>
 static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
     auto kernel = mid_gemm_kernel<RGW, MH, DEPTH, WN, DX>;
-    static size_t granted[16] = {};
+    static LdsGranted granted;
     if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
     kernel<<<dim3(grid), dim3(WN * 128), lds, stream>>>(a);
     return report_hip("mid_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;

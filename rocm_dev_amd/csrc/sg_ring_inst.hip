@@ -12,7 +12,7 @@ namespace sg {
 template <int BL, int XU>
 static int launch_one(int nt, const RingArgs& ra, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
     auto kernel = nt ? ring_gemm_kernel<SG_MT, BL, XU, true> : ring_gemm_kernel<SG_MT, BL, XU, false>;
-    static size_t granted[2][16] = {};
+    static LdsGranted granted[2];
     if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted[nt ? 1 : 0])) return rc;
     kernel<<<dim3(grid), dim3(threads), lds, stream>>>(ra);
     return report_hip("ring_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;

@@ -9,7 +9,7 @@ template <int MT, int RG, int XU2, int DEPTH>
 static int launch_one(const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
     if (threads > (unsigned)sparse_launch_bound(MT, RG)) return SG_INVALID_CONFIG;
     auto kernel = sparse24_gemm_kernel<MT, RG, XU2, DEPTH>;
-    static size_t granted[16] = {};
+    static LdsGranted granted;
     if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
     kernel<<<dim3(grid), dim3(threads), lds, stream>>>(sa);
     return report_hip("sparse24_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;

@@ -8,7 +8,7 @@ template <int MT, int RG, int PT, int DEPTH>
 static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
     if (threads > (unsigned)xreg_launch_bound(MT, RG, PT)) return SG_INVALID_CONFIG;
     auto kernel = lds_gemm_xreg_kernel<MT, RG, PT, DEPTH, true>;
-    static size_t granted[16] = {};
+    static LdsGranted granted;
     if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
     kernel<<<dim3(grid), dim3(threads), lds, stream>>>(a);
     return report_hip("lds_gemm_xreg_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
