@@ -409,7 +409,10 @@ def test_mid_batch_engine(sg, oracle, cfg, shape):
 
 
 @pytest.mark.parametrize("m,n,k", [(64, 10240, 8192), (128, 10240, 8192), (128, 8192, 8192), (256, 8192, 8192),
-                                   (128, 57344, 8192), (256, 57344, 8192), (64, 8192, 28672), (256, 8192, 28672)])
+                                   (64, 57344, 8192), (128, 57344, 8192), (256, 57344, 8192), (64, 8192, 28672),
+                                   (256, 8192, 28672),
+                                   # 224-row tiles with ragged m and few K blocks (the rotated K start wraps within 8 or 24)
+                                   (33, 57344, 1024), (50, 57344, 3072), (100, 57344, 1024), (200, 57344, 3072)])
 def test_mid_batch_config4_shapes(sg, oracle, m, n, k):
     """benchmark configuration 4 shapes at full size through the fastpath.  The oracle checks two
     512-row slices of the weight matrix (tiles are independent along n); the rest is covered
@@ -430,7 +433,7 @@ def test_mid_batch_config4_shapes(sg, oracle, m, n, k):
     for lo in (0, n - 512):
         b8 = B[lo:lo + 512].cpu().numpy()
         ref = oracle.gemm_omp(a8, b8, scale)
-        assert oracle.max_rel_err_bf16(got[:, lo:lo + 512], ref) <= GEMM_TOL
+        assert oracle.max_rel_err_bf16(got[:, lo:lo + 512], ref) <= gemm_tol(k)
     D2 = torch.empty_like(D)
     assert sg.skinny_gemm_fastpath(A, B, D2, scale_tensor(2 * scale)) == 0
     torch.cuda.synchronize()
