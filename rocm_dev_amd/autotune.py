@@ -239,10 +239,14 @@ def agrees(d, ref, tol=1e-2):
     return bool(((d - ref).abs() / ref.abs().clamp_min(floor)).max() <= tol)
 
 
-def tune_shape(m, n, k, top=1, launches=20, verbose=False, limit=None):
-    """Times every candidate of the shape; returns [(us, record)] sorted, fastest first, candidates whose
-    result disagrees with the library's default choice excluded, and the default's own time."""
-    import ctypes as C  # noqa: F401
+def tune_shape(m, n, k, top=1, launches=20, verbose=False, limit=None, finalists=8, rounds=3):
+    """Times every candidate of the shape once, then the `finalists` fastest and the library's own choice again in
+    `rounds` alternating rounds (one timing after another is repeatable to a few per cent only: the first graphs of
+    a process run slow and clocks drift; alternating rounds repeat to a few parts per thousand).  Returns
+    ([(us, record)] fastest first by the median over the rounds, candidates whose result disagrees with the
+    library's default choice excluded; the default's median; candidates that ran)."""
+    import statistics
+
     from ._lib import lib
     from .api import SgTuning
     bench = Bench(m, n, k)
@@ -250,29 +254,33 @@ def tune_shape(m, n, k, top=1, launches=20, verbose=False, limit=None):
     ref = bench.result(lib, default)
     if ref is None:
         raise RuntimeError("the library rejects shape %dx%dx%d" % (m, n, k))
-    base_us = bench.time(lib, default, launches)
+    bench.time(lib, default, launches)          # warm-up: the first timed graph of a process is not representative
     timed = []
     space = search_space(m, n, k)
     if limit:
         space = space[:limit]
     for r in space:
-        t = SgTuning(*(r[f] for f in FIELDS))
-        us = bench.time(lib, t, launches)
+        us = bench.time(lib, SgTuning(*(r[f] for f in FIELDS)), launches, repeats=2)
         if us is None:
             continue
         timed.append((us, r))
     timed.sort(key=lambda e: e[0])
-    base_us = min(base_us, bench.time(lib, default, launches))   # again at the end: clocks and caches have settled
     kept = []
-    for us, r in timed:                      # verify only as many as are reported
+    for us, r in timed:                      # verify only as many as go into the final rounds
         d = bench.result(lib, SgTuning(*(r[f] for f in FIELDS)))
         if d is not None and agrees(d, ref):
-            kept.append((us, r))
+            kept.append(r)
         elif verbose:
             print("  dropped (result differs): %s" % (r,), file=sys.stderr)
-        if len(kept) >= top:
+        if len(kept) >= max(top, finalists):
             break
-    return kept, base_us, len(timed)
+    base, samples = [], [[] for _ in kept]
+    for _ in range(max(1, rounds)):
+        base.append(bench.time(lib, default, launches))
+        for i, r in enumerate(kept):
+            samples[i].append(bench.time(lib, SgTuning(*(r[f] for f in FIELDS)), launches))
+    final = sorted(((statistics.median(v), r) for v, r in zip(samples, kept)), key=lambda e: e[0])
+    return final[:top], statistics.median(base), len(timed)
 
 
 def main(argv=None):
