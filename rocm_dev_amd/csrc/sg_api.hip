@@ -387,13 +387,27 @@ static int launch_sparse_engine(const Config& c, StreamArgs a, const uint8_t* me
         const int need = (a.m + 3) / 4;
         xu2 = need <= 1 ? 2 : (need <= 2 ? 4 : 8);
     }
+    SparseArgs sa;
+    sa.meta = meta;
+    if (c.wavetile == 1) {
+        // every wave owns whole tiles, the activation matrix is resident in LDS: one activation tile of at most 16
+        // rows, no K split, c.persist workgroups per CU at most
+        if (c.mt != 1 || a.m_tiles != 1 || c.split_k != 1 || c.persist < 1 || (c.rg != 1 && c.rg != 2)) return SG_INVALID_CONFIG;
+        if (c.waves * 64 > 1024) return SG_TOO_MANY_WARPS;
+        const size_t lds_wt = (size_t)(a.k / 512) * xu2 * 1024 + (size_t)c.waves * c.depth * c.rg * 5120 + 8192;
+        if (lds_wt > 159 * 1024) return SG_INVALID_CONFIG;
+        DeviceInfo* dev;
+        if (int rc = get_device_info(&dev)) return rc;
+        size_t grid = (size_t)dev->cu_count * c.persist;
+        if (grid > tiles) grid = tiles;
+        sa.g = a;
+        return launch_sparse_wavetile(c.rg, xu2, c.depth, sa, (unsigned)grid, (unsigned)c.waves * 64, lds_wt, stream);
+    }
     const size_t stage = (size_t)(c.rg * 5 + xu2) * 1024;
     // + 8 KB: lanes of activation rows that are not loaded read past the last slot
     const size_t lds = (size_t)c.waves * c.depth * stage + 8192;
     if (lds > 159 * 1024) return SG_INVALID_CONFIG;
-    SparseArgs sa;
     sa.g = a;
-    sa.meta = meta;
     return launch_sparse(c.mt, c.rg, xu2, c.depth, sa, (unsigned)(tiles * c.split_k), (unsigned)c.waves * 64, lds, stream);
 }
 
@@ -417,6 +431,21 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
     while (c.depth > 2 && ((c.depth - 1) * (c.rg * 5 + xu2) > 63 ||
                            (size_t)c.waves * c.depth * (c.rg * 5 + xu2) * 1024 + 8192 > 159 * 1024))
         c.depth--;
+    if (c.mt == 1 && m > 4 && tiles16 * 4 >= cu_count * 5) {
+        // 5..16 activation rows and more than one tile per CU: the activation matrix stays resident in LDS and
+        // four waves per CU each stream whole tiles (4-33 % faster on ten shapes than refetching 4-8 KB of
+        // activations with every 5 KB weight stage; at four rows and below the two are level)
+        const size_t x_res = (size_t)(k / 512) * xu2 * 1024;
+        for (int depth = 4; depth >= 2; depth--) {
+            if (x_res + (size_t)4 * depth * 5120 + 8192 > 159 * 1024) continue;
+            c.rg = 1;
+            c.waves = 4;
+            c.depth = depth;
+            c.persist = 1;
+            c.wavetile = 1;
+            break;
+        }
+    }
     return c;
 }
 
@@ -937,7 +966,10 @@ int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_
         c.depth = t->depth;
         c.split_k = t->split_k;
         c.mt = t->m_blocks;
+        c.persist = t->persistent_wgs_per_cu;
+        c.wavetile = t->wave_tiles;
         if (c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
+        if (c.wavetile != 0 && c.wavetile != 1) return SG_INVALID_CONFIG;
     }
     StreamArgs a{};
     a.A = A; a.B = B_vals; a.D = D; a.scale = scale_tensor;

@@ -33,4 +33,26 @@ int launch_sparse(int mt, int rg, int xu2, int depth, const SparseArgs& sa, unsi
     return SG_INVALID_CONFIG;
 }
 
+template <int RG, int XU2, int DEPTH>
+static int launch_wavetile(const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
+    if (threads > (RG == 4 ? 512u : 1024u)) return SG_INVALID_CONFIG;
+    auto kernel = sparse24_gemm_wavetile_kernel<RG, XU2, DEPTH>;
+    static LdsGranted granted;
+    if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
+    kernel<<<dim3(grid), dim3(threads), lds, stream>>>(sa);
+    return report_hip("sparse24_gemm_wavetile_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
+}
+
+#define SG_WT_CASE(RG_, XU2_, DEPTH_)                                                                  \
+    if (rg == RG_ && xu2 == XU2_ && depth == DEPTH_) return launch_wavetile<RG_, XU2_, DEPTH_>(sa, grid, threads, lds, stream);
+#define SG_WT_DEPTHS(RG_, XU2_) SG_WT_CASE(RG_, XU2_, 2) SG_WT_CASE(RG_, XU2_, 3) SG_WT_CASE(RG_, XU2_, 4) SG_WT_CASE(RG_, XU2_, 6)
+
+// wave-per-tile kernel with the activations resident in LDS (at most 16 activation rows)
+int launch_sparse_wavetile(int rg, int xu2, int depth, const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds,
+                           hipStream_t stream) {
+    SG_WT_DEPTHS(1, 2) SG_WT_DEPTHS(1, 4) SG_WT_DEPTHS(1, 8)
+    SG_WT_DEPTHS(2, 2) SG_WT_DEPTHS(2, 4) SG_WT_DEPTHS(2, 8)
+    return SG_INVALID_CONFIG;
+}
+
 }  // namespace sg

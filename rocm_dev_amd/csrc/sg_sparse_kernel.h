@@ -174,4 +174,154 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
     finish_tile<RG, MT>(a, acc, reinterpret_cast<f32x4*>(ring), &arrival, tile_m, tile_n, split, m0, n0);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Wave-per-tile variant with the activations resident in LDS, for many weight rows and at most 16
+// activation rows (the up-projection of a sparse MLP at decode batch sizes).  Next to a 16-row stage of
+// compressed weights (5 KB) the activations of the same 512 k are 2-8 KB, so in the kernel above up to
+// 60 % of what a workgroup pulls through L2 is the same activation matrix over and over.  Here a workgroup
+// fetches the activation matrix once, every wave owns whole 16*RG-row tiles over the full K range - no
+// cross-wave reduction, no barrier after the prologue - and its ring carries weights only and runs on across
+// tile boundaries.  Tiles are dealt to workgroups first (wave w of workgroup b owns tiles b + G*w,
+// b + G*(w + W), ...), so that with three or four tiles per CU every CU streams; every wave starts its
+// tiles at a K stage of its own and wraps (waves in step at one K offset load the memory channels unevenly).
+template <int RG, int XU2, int DEPTH>
+__global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_kernel(const SparseArgs sa) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // X[stages][XU2 KB] | [wave][DEPTH][RG*5 KB] | 8 KB
+    const StreamArgs& a = sa.g;
+
+    constexpr int PER_STAGE = RG * 5;
+    constexpr int STAGE_BYTES = PER_STAGE * 1024;
+    static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
+
+    const int lane = lane_id();
+    const int wave = wave_id();
+    const int waves = a.waves;
+    const int blocks = a.k >> 9;   // 512-k stages
+    const int first = (int)blockIdx.x + (int)gridDim.x * wave;
+    const int stride = (int)gridDim.x * waves;
+    const int my_tiles = first < a.n_tiles ? (a.n_tiles - first + stride - 1) / stride : 0;
+    const int total = blocks * my_tiles;
+    const int k_rot = (int)(((unsigned)blockIdx.x * (unsigned)waves + (unsigned)wave) % (unsigned)blocks);
+    auto rotated = [&](int kb) __attribute__((always_inline)) { return kb + k_rot >= blocks ? kb + k_rot - blocks : kb + k_rot; };
+
+    const int v_row = lane >> 4, v_pp = lane & 15;     // values / activations: 4 rows x 16 pieces
+    const int t_row = lane >> 2, t_pp = lane & 3;      // metadata: 16 rows x 4 pieces
+    const size_t v_stride = (size_t)(a.k >> 1), t_stride = (size_t)(a.k >> 3);
+    const int x_bytes = blocks * XU2 * 1024;
+    const uint8_t* my_ring = ring + x_bytes + (size_t)wave * (DEPTH * STAGE_BYTES);
+    const unsigned my_ring_lds = lds_addr(my_ring);
+    const unsigned x_lds = lds_addr(ring);
+
+    // ---- resident activations: stage kb is fetched by wave kb % waves, in the layout of a stage's activation part
+    int x_issued = 0;
+    for (int kb = wave; kb < blocks; kb += waves) {
+#pragma unroll
+        for (int i = 0; i < XU2; i++) {
+            const int row_l = 4 * (i >> 1) + v_row;
+            const int row = row_l < a.m ? row_l : a.m - 1;
+            dma_1kb(a.A + (size_t)row * a.k + ((size_t)kb << 9) + (i & 1) * 256 + ((v_pp ^ (row_l & 15)) << 4),
+                    x_lds + (unsigned)(kb * XU2 + i) * 1024);
+        }
+        x_issued += XU2;
+    }
+
+    auto issue = [&](int i) __attribute__((always_inline)) {
+        const int j = i / blocks;
+        const size_t kb = (size_t)rotated(i - j * blocks);
+        const int n0 = (first + j * stride) * (16 * RG);
+        const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int row16 = 4 * u + v_row;
+                int row = n0 + rg * 16 + row16;
+                row = row < a.n ? row : a.n - 1;   // past the edge: re-read the last row, never stored
+                dma_1kb_stream(a.B + (size_t)row * v_stride + ((v_pp ^ row16) << 4) + (kb << 8), slot + (rg * 5 + u) * 1024);
+            }
+            int row = n0 + rg * 16 + t_row;
+            row = row < a.n ? row : a.n - 1;
+            dma_1kb_stream(sa.meta + (size_t)row * t_stride + ((t_pp ^ (t_row >> 2)) << 4) + (kb << 6), slot + (rg * 5 + 4) * 1024);
+        }
+    };
+
+    const int r = lane & 15, g = lane >> 4;
+    const int v_rd = (r >> 2) * 1024 + (r & 3) * 256;
+    const int t_rd = 4096 + r * 64 + ((g ^ (r >> 2)) << 4);
+    const int x_rd = ((r >> 2) * 2 + (g >> 1)) * 1024 + (r & 3) * 256;
+
+    f32x4 acc[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) acc[rg] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    int kb_cur = 0;   // stages of the current tile already consumed
+    auto consume = [&](int i) __attribute__((always_inline)) {
+        const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES;
+        const uint8_t* xs = ring + (size_t)rotated(kb_cur) * (XU2 * 1024);
+        i32x4 x[8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) x[t] = *reinterpret_cast<const i32x4*>(xs + x_rd + (((8 * (g & 1) + t) ^ r) << 4));
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const uint8_t* w = slot + rg * 5120;
+            const i32x4 idx = *reinterpret_cast<const i32x4*>(w + t_rd);
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+                const i32x4 v = *reinterpret_cast<const i32x4*>(w + v_rd + (((4 * g + p) ^ r) << 4));
+                const i32x2 v_lo = {v.x, v.y}, v_hi = {v.z, v.w};
+                const int id_lo = idx[p] & 0xffff, id_hi = (unsigned)idx[p] >> 16;
+                acc[rg] = __builtin_amdgcn_smfmac_f32_16x16x64_fp8_fp8(v_lo, x[2 * p], acc[rg], id_lo, 0, 0);
+                acc[rg] = __builtin_amdgcn_smfmac_f32_16x16x64_fp8_fp8(v_hi, x[2 * p + 1], acc[rg], id_hi, 0, 0);
+            }
+        }
+    };
+
+    const float scale = a.scale ? a.scale[0] : 1.0f;
+    int tile_j = 0;
+    auto after_consume = [&]() __attribute__((always_inline)) {
+        if (++kb_cur == blocks) {   // the tile is complete: scale, round, store, start the next one
+            kb_cur = 0;
+            const int n0 = (first + tile_j * stride) * (16 * RG);
+            tile_j++;
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                store_fragment(a, acc[rg], scale, r, n0 + rg * 16 + 4 * g);
+                acc[rg] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+    };
+
+    // weight prologue behind the activations; once at most pro * PER_STAGE DMAs are outstanding this wave's share of
+    // the activations has landed, and the barrier publishes everyone's
+    const int pro = total < DEPTH ? total : DEPTH;
+    for (int d = 0; d < pro; d++) issue(d);
+    if (x_issued > 0) wait_vmcnt_upto(pro * PER_STAGE);
+    __syncthreads();
+
+    if (total >= DEPTH) {
+        int i = 0;
+        for (; i + DEPTH < total; i++) {
+            wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            consume(i);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            issue(i + DEPTH);
+            __builtin_amdgcn_sched_barrier(0);
+            after_consume();
+        }
+        auto consume_and_close = [&](int ii) __attribute__((always_inline)) {
+            consume(ii);
+            after_consume();
+        };
+        drain_ring<0, DEPTH, PER_STAGE>(consume_and_close, i);
+    } else {
+        wait_vmcnt<0>();
+        for (int i = 0; i < total; i++) {
+            consume(i);
+            after_consume();
+        }
+    }
+}
+
+
 }  // namespace sg

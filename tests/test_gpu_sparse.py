@@ -88,6 +88,48 @@ def test_sparse_tuned_configs(sg, oracle, cfg, shape):
     assert rc == 0 and np.array_equal(again, got)
 
 
+WAVETILE_CONFIGS = [
+    # waves, row_tiles, depth, workgroups per CU
+    (4, 1, 4, 1),
+    (1, 1, 2, 1),
+    (8, 1, 3, 1),
+    (3, 2, 3, 1),
+    (4, 2, 6, 2),
+    (16, 1, 2, 1),
+]
+
+
+@pytest.mark.parametrize("cfg", WAVETILE_CONFIGS)
+@pytest.mark.parametrize("shape", [(8, 14336, 4096), (1, 4096, 1024), (5, 1000, 1024), (16, 6000, 2048), (13, 200, 512),
+                                   (3, 34, 3584)])
+def test_sparse_wave_per_tile_configs(sg, oracle, cfg, shape):
+    """The wave-per-tile kernel (activations resident in LDS, every wave a whole tile over all of K, rotated K start):
+    more tiles than waves, fewer tiles than waves, ragged n and m, a single K stage, a K range of seven stages."""
+    waves, row_tiles, depth, per_cu = cfg
+    m, n, k = shape
+    a8, vals, meta, b8, scale = oracle.make_sparse24_operands(m, n, k, seed=33)
+    ref = oracle.gemm_sparse24(a8, vals, meta, scale)
+    t = sg.SgTuning(2, 1, waves, row_tiles, 1, depth, 8, 1, per_cu, 1)
+    rc, got = _run(sg, a8, vals, meta, scale, tuning=t)
+    if rc == 6:
+        pytest.skip("configuration not compiled / does not fit LDS")
+    assert rc == 0, sg.strerror(rc)
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
+    rc, again = _run(sg, a8, vals, meta, scale, tuning=t)
+    assert rc == 0 and np.array_equal(again, got)
+
+
+def test_sparse_wave_per_tile_rejects_what_it_cannot_run(sg, oracle):
+    a8, vals, meta, b8, scale = oracle.make_sparse24_operands(24, 256, 1024, seed=1)
+    for t in (sg.SgTuning(2, 1, 4, 1, 2, 2, 8, 1, 1, 1),      # two activation blocks do not fit next to the rings
+              sg.SgTuning(2, 2, 4, 1, 1, 2, 8, 1, 1, 1),      # no K split
+              sg.SgTuning(2, 1, 4, 1, 1, 2, 8, 1, 0, 1),      # needs a workgroup count per CU
+              sg.SgTuning(2, 1, 4, 4, 1, 2, 8, 1, 1, 1),      # row_tiles 1 or 2
+              sg.SgTuning(2, 1, 4, 1, 1, 2, 8, 1, 1, 2)):     # unknown mode
+        rc, _ = _run(sg, a8[:t.m_blocks * 16 if t.m_blocks == 2 else 8], vals, meta, scale, tuning=t)
+        assert rc == 6, (rc, [getattr(t, f) for f, _ in t._fields_])
+
+
 @pytest.mark.parametrize("n,k", [(4096, 14336), (14336, 4096)])
 @pytest.mark.parametrize("m", [1, 8, 16, 32])
 def test_config5_shapes(sg, oracle, m, n, k):
