@@ -186,7 +186,9 @@ int sg_async_gemm_bf16(const uint8_t* A, const uint8_t* B, void* D_bf16, int m, 
  * k must be a multiple of 512, n even; all pointers 16-byte aligned.  The weights are the
  * sparse operand of gfx950's v_smfmac_f32_16x16x64_fp8_fp8; HBM traffic is 0.625 bytes per
  * dense weight.  The _tuned form takes row_tiles, waves, depth, split_k and m_blocks from
- * the record (engine 0 = library's choice). */
+ * the record (engine 0 = library's choice); wave_tiles = 1 with persistent_wgs_per_cu >= 1
+ * selects the kernel that keeps the activation matrix resident in LDS and gives every wave
+ * whole 16*row_tiles-row tiles (m <= 16, split_k = 1, row_tiles 1 or 2). */
 int sg_sparse24_gemm(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D_bf16,
                      const float* scale_tensor, int m, int n, int k, void* stream);
 int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D_bf16,
