@@ -50,7 +50,7 @@ def test_one_hot_metadata_positions(sg, oracle):
 
 
 @pytest.mark.parametrize("m", [1, 3, 8, 13, 16, 27, 32])
-@pytest.mark.parametrize("n,k", [(64, 512), (1000, 1024), (512, 4096)])
+@pytest.mark.parametrize("n,k", [(64, 512), (1000, 1024), (512, 4096), (6002, 1536)])   # the last: more than one tile per CU
 def test_sparse_small(sg, oracle, m, n, k):
     a8, vals, meta, b8, scale = oracle.make_sparse24_operands(m, n, k, seed=m)
     ref = oracle.gemm_sparse24(a8, vals, meta, scale)
