@@ -59,6 +59,11 @@ def main():
                     help="only launch the decode-sweep GEMMs (four projection shapes x M = 1, 8, 32), eagerly, three "
                          "times each on cold weights, after three 256 MiB copies of known traffic, and exit "
                          "(for HBM-traffic counter runs; prints no JSON line)")
+    ap.add_argument("--sparse-counters", action="store_true",
+                    help="only launch the 2:4 GEMMs (14336 x 4096 and 28672 x 4096 at M = 8, 16), eagerly, three times each "
+                         "on cold weights through the library's choice and three times through the one-wave-workgroup kernel "
+                         "it replaced, after three 256 MiB copies of known traffic, and exit (for L2 / HBM traffic counter runs; "
+                         "prints no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1")
@@ -94,6 +99,43 @@ def main():
                         raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
                 torch.cuda.synchronize()
             del wb
+        return
+
+    if args.sparse_counters:
+        import ctypes
+        one = torch.ones(1, device="cuda")
+        src = torch.empty(256 << 20, device="cuda", dtype=torch.uint8)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        for (n, k) in ((14336, 4096), (28672, 4096)):
+            copies = 6
+            vb, mb = [], []
+            for _ in range(copies):
+                dense = torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8)
+                v = torch.empty((n, k // 2), device="cuda", dtype=torch.uint8)
+                t = torch.empty((n, k // 8), device="cuda", dtype=torch.uint8)
+                if lib.sg_sparse24_compress(dense.data_ptr(), v.data_ptr(), t.data_ptr(), n, k, k, None) != 0:
+                    raise RuntimeError("sg_sparse24_compress failed")
+                vb.append(v)
+                mb.append(t)
+            del dense
+            torch.cuda.synchronize()
+            for m in (8, 16):
+                a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+                d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+                # engine 0: the library's choice (wave-per-tile, activations resident in LDS);
+                # then one-wave workgroups with the activations in every stage, two ring slots
+                for rec in (sg.SgTuning(0, 1, 1, 1, 1, 2, 8, 1, 0, 0), sg.SgTuning(2, 1, 1, 1, 1, 2, 8, 1, 0, 0)):
+                    for i in range(3):
+                        rc = lib.sg_sparse24_gemm_tuned(a8.data_ptr(), vb[(3 * (m // 8) + i) % copies].data_ptr(),
+                                                        mb[(3 * (m // 8) + i) % copies].data_ptr(), d.data_ptr(), one.data_ptr(),
+                                                        m, n, k, ctypes.byref(rec), None)
+                        if rc != 0:
+                            raise RuntimeError("sg_sparse24_gemm_tuned: %s" % sg.strerror(rc))
+                    torch.cuda.synchronize()
+            del vb, mb
         return
 
     if args.mid_batch_counters:
