@@ -168,9 +168,8 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         lds = (size_t)(a.k / 256) * xu * 1024 + (size_t)c.waves * c.depth * c.rg * 4096 + 4096;
         DeviceInfo* dev;
         if (int rc = get_device_info(&dev)) return rc;
-        size_t want = (tiles + c.waves - 1) / c.waves;
-        const size_t cap = (size_t)dev->cu_count * c.persist;
-        if (want > cap) want = cap;
+        size_t want = (size_t)dev->cu_count * c.persist;
+        if (want > tiles) want = tiles;
         grid = (unsigned)want;
     } else if (c.persist > 0 && (c.wavetile & 3) == 3) {
         // activations resident in registers: every wave keeps the fragments of its own K blocks
@@ -480,8 +479,9 @@ static Config pick_config(int m, int n, int k, int cu_count) {
         c.ku = 4;
         const int blocks = k / 256;
         const int xu0 = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
-        if (tiles16 >= 2 * cu_count) {
-            // several tiles per CU: one persistent workgroup per CU walks them with continuous rings;
+        if (c.mt == 2 ? tiles16 >= 2 * cu_count : tiles16 > 2 * cu_count) {
+            // more than two tiles per CU (at exactly two, one-wave workgroups are still 2-3 % ahead up to 16 rows;
+            // at 2.25 they are 20 % behind): one persistent workgroup per CU walks them with continuous rings;
             // when one activation tile covers all of m, it stays resident in LDS and the stages
             // carry weights only
             c.rg = 1;

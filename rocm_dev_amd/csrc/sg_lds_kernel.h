@@ -433,7 +433,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
 // so there is no cross-wave reduction and no barrier after the prologue.  The whole activation
 // matrix (ceil(m/4) KB per 256-byte K block) is fetched once per workgroup and shared by its
 // waves, which removes a third of the DMA instructions and of the L2 traffic at m = 8.  Wave
-// (workgroup b, wave w) walks tiles b*W + w, + total waves, ...; its weight ring runs across
+// (workgroup b, wave w) walks tiles b + G*w, + total waves, ...; its weight ring runs across
 // tile boundaries.
 template <int MT, int RG, int XU, int DEPTH, bool NT>
 __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_wavetile_kernel(const StreamArgs a) {
@@ -452,10 +452,13 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
 
     const int blocks = a.k >> 8;
     const int total_tiles = a.n_tiles * a.m_tiles;
+    // tiles are dealt to workgroups first (wave w of workgroup b owns tiles b + G*w, b + G*(w + W), ...), so that a
+    // few tiles per CU still put a stream on every CU
     const int total_waves = (int)gridDim.x * waves;
-    const int gw = (int)blockIdx.x * waves + wave;
-    const int my_tiles = gw < total_tiles ? (total_tiles - gw + total_waves - 1) / total_waves : 0;
+    const int first = (int)blockIdx.x + (int)gridDim.x * wave;
+    const int my_tiles = first < total_tiles ? (total_tiles - first + total_waves - 1) / total_waves : 0;
     const int total = blocks * my_tiles;
+    const int gw = (int)blockIdx.x * waves + wave;   // for the K rotation: neighbours in a workgroup start one block apart
     // Every wave starts its tiles at a different K block and wraps around.  Here all waves of the chip would
     // otherwise ask for block kb of their rows at the same moment, and row pitches are multiples of 4 KB: in step,
     // 8 x 28672 x 4096 takes 24.6 us, spread over all K offsets 19.6 us (eight waves, same process, interleaved).
@@ -489,7 +492,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
         const int j = i / blocks;
         int kb = i - j * blocks + k_rot;
         kb = kb >= blocks ? kb - blocks : kb;
-        const int n0 = ((gw + j * total_waves) % a.n_tiles) * (16 * RG);
+        const int n0 = ((first + j * total_waves) % a.n_tiles) * (16 * RG);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
         const size_t koff = ((size_t)kb << 8) + src_col;
 #pragma unroll
@@ -522,7 +525,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     auto after_consume = [&]() __attribute__((always_inline)) {
         if (++kb_cur == blocks) {   // the tile is complete: scale, round, store, start the next one
             kb_cur = 0;
-            const int n0 = ((gw + tile_j * total_waves) % a.n_tiles) * (16 * RG);
+            const int n0 = ((first + tile_j * total_waves) % a.n_tiles) * (16 * RG);
             tile_j++;
 #pragma unroll
             for (int f = 0; f < FRAGS; f++) {
