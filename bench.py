@@ -391,6 +391,16 @@ def main():
                             "TFLOPs": round(2.0 * m * n * k / us / 1e6, 1), "frac_fp8_peak": round(2.0 * m * n * k / us / 1e6 / 5000.0, 4)})
             del wb
         others["mid_batch"] = mid
+        # fp32 batch sum D = sum_b (A_b + B_b): what the reference's split-K experiments reduce their partials with
+        tb, tm, tn = 8, 1024, 8192
+        ta = torch.randn((tb, tm, tn), device="cuda", dtype=torch.float32)
+        tbb = torch.randn((tb, tm, tn), device="cuda", dtype=torch.float32)
+        td = torch.empty((tm, tn), device="cuda", dtype=torch.float32)
+        tsr_us = graph_time_us(lambda i, st: lib.sg_tiled_sum_reduce(ta.data_ptr(), tbb.data_ptr(), td.data_ptr(), tb, tm, tn, st), 8)
+        tsr_bytes = (2 * tb + 1) * tm * tn * 4
+        others["tiled_sum_reduce_8x1024x8192"] = {"us": round(tsr_us, 2), "TBps": round(tsr_bytes / tsr_us / 1e6, 3),
+                                                  "note": "reads 512 MiB per launch (beyond the 256 MB cache), writes 32 MiB"}
+        del ta, tbb, td
         # 2:4 sparse GEMMs
         sp = []
         for (n, k) in ((4096, 14336), (14336, 4096)):

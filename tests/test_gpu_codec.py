@@ -124,7 +124,10 @@ def test_full_size_properties(sg, oracle):
         assert np.array_equal(S[sl].cpu().numpy(), s_ref)
 
 
-@pytest.mark.parametrize("b,m,n", [(1, 8, 64), (5, 8, 64), (9, 24, 192), (3, 7, 33), (16, 128, 1024)])
+@pytest.mark.parametrize("b,m,n", [(1, 8, 64), (5, 8, 64), (9, 24, 192), (3, 7, 33), (16, 128, 1024),
+                                   # 32 KB per workgroup and stream from 4 M elements on: whole workgroups, a ragged
+                                   # last one, and an element count that is not a multiple of four
+                                   (8, 512, 8192), (3, 2049, 2052), (2, 2051, 2051)])
 def test_tiled_sum_reduce(sg, oracle, b, m, n):
     A = oracle.uniform_f32((b, m, n), 0, 7, -0.5, 0.5)
     B = oracle.uniform_f32((b, m, n), 0, 8, -0.5, 0.5)
