@@ -19,8 +19,8 @@ namespace sg {
 template <int CH>
 __global__ void __launch_bounds__(256) tiled_sum_reduce_kernel(const float* __restrict__ A, const float* __restrict__ B,
                                                                float* __restrict__ D, int b, size_t mn) {
-    const size_t base = (size_t)blockIdx.x * (1024 * CH) + threadIdx.x * 4;
     if ((mn & 3) == 0 && (size_t)(blockIdx.x + 1) * (1024 * CH) <= mn) {
+        const size_t base = (size_t)blockIdx.x * (1024 * CH) + threadIdx.x * 4;
         f32x4 acc[CH];
 #pragma unroll
         for (int c = 0; c < CH; c++) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -39,13 +39,16 @@ __global__ void __launch_bounds__(256) tiled_sum_reduce_kernel(const float* __re
 #pragma unroll
         for (int c = 0; c < CH; c++) *reinterpret_cast<f32x4*>(D + base + c * 1024) = acc[c];
     } else {
-        // the last, partial workgroup, or m*n not a multiple of four: element by element
-        for (int c = 0; c < CH; c++)
-            for (size_t i = base + (size_t)c * 1024; i < mn && i < base + (size_t)c * 1024 + 4; i++) {
-                float acc = 0.f;
-                for (int ib = 0; ib < b; ib++) acc = __fadd_rn(acc, __fadd_rn(A[(size_t)ib * mn + i], B[(size_t)ib * mn + i]));
-                D[i] = acc;
-            }
+        // the last, partial workgroup, or m*n not a multiple of four (batches then start at unaligned addresses):
+        // one float per lane and step, neighbouring lanes on neighbouring floats
+        const size_t first = (size_t)blockIdx.x * (1024 * CH) + threadIdx.x;
+        for (int j = 0; j < 4 * CH; j++) {
+            const size_t i = first + (size_t)j * 256;
+            if (i >= mn) break;
+            float acc = 0.f;
+            for (int ib = 0; ib < b; ib++) acc = __fadd_rn(acc, __fadd_rn(A[(size_t)ib * mn + i], B[(size_t)ib * mn + i]));
+            D[i] = acc;
+        }
     }
 }
 
