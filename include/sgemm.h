@@ -51,11 +51,19 @@ typedef enum SgReturnCode {
 
 const char* sg_strerror(int code);
 
-/* Library-owned split-K workspace, one per device, created on first use by a launcher
- * that needs it (split_k > 1).  sg_init() creates it eagerly for the current device so
- * that later launches allocate nothing.  Two launches that use split-K concurrently on
- * different streams of one device share it and therefore must not overlap. */
+/* Library-owned split-K workspaces (fp32 partial fragments + one arrival counter per output tile), one per
+ * device and stream: launches on one stream run in order and share a workspace, launches on different
+ * streams may overlap and never share one.  A workspace is created, or grown, by the first launch on its
+ * stream that needs it (split_k > 1, also when the library chooses the split itself); at most 512 MB of
+ * partials per launch, beyond that SG_WORKSPACE_TOO_SMALL.  An outgrown buffer is kept until the process
+ * ends.  A launch recorded into a HIP graph keeps the workspace of the stream it was captured on: run no
+ * other split-K work on that stream while the graph replays elsewhere.
+ *   sg_init          sets up the current device and a 64 MB workspace for the default stream
+ *   sg_init_stream   the same for `stream` with room for partial_bytes of partials, so that later launches
+ *                    on it allocate nothing
+ *   sg_workspace_bytes  device memory the workspaces of the current device hold */
 int    sg_init(void);
+int    sg_init_stream(void* stream, size_t partial_bytes);
 size_t sg_workspace_bytes(void);
 
 /*

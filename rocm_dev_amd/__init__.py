@@ -21,6 +21,8 @@ from .api import (  # noqa: F401
     skinny_gemm_pick,
     skinny_gemm_rowcol,
     skinny_gemm_tuned,
+    init_stream,
+    workspace_bytes,
     strerror,
     tiled_sum_reduce,
     tuning_clear,

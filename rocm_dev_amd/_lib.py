@@ -19,6 +19,7 @@ _vp, _i, _sz = C.c_void_p, C.c_int, C.c_size_t
 SIGNATURES = {
     "sg_strerror": (C.c_char_p, [_i]),
     "sg_init": (_i, []),
+    "sg_init_stream": (_i, [_vp, _sz]),
     "sg_workspace_bytes": (_sz, []),
     "sg_skinny_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm_fastpath": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),

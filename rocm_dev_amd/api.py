@@ -135,6 +135,16 @@ def skinny_gemm_tuned(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k=1, wave
     return _done(rc, check)
 
 
+def init_stream(stream=None, partial_bytes=64 << 20, check=True):
+    """Create the split-K workspace of `stream` (torch stream; None = torch's current stream) ahead of time."""
+    handle = _stream() if stream is None else stream.cuda_stream
+    return _done(lib.sg_init_stream(handle, partial_bytes), check)
+
+
+def workspace_bytes():
+    return lib.sg_workspace_bytes()
+
+
 def skinny_gemm_pick(m, n, k):
     """The tunables the fastpath would use: dict with the reference's parameter names."""
     out = (C.c_int * 8)()

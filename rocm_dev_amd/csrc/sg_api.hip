@@ -25,11 +25,17 @@ int launch_sparse24_compress(const uint8_t* B, uint8_t* vals, uint8_t* meta, int
 
 // ---- per-device state -------------------------------------------------------------------
 constexpr int kMaxDevices = 16;
-constexpr size_t kPartialBytes = 64u << 20;  // fp32 split-K partials
-constexpr size_t kCounters = 1u << 18;       // arrival counters (one per output tile)
+constexpr size_t kDefaultPartialBytes = 64u << 20;  // what sg_init() sets up for the default stream
+constexpr size_t kMinPartialBytes = 4u << 20;       // smallest partials buffer created on demand
+constexpr size_t kMaxPartialBytes = 512u << 20;     // one launch may not ask for more
+constexpr size_t kMinCounters = 1u << 14;           // arrival counters (one per output tile)
+constexpr size_t kMaxCounters = 1u << 22;
 
 static std::mutex g_mutex;
-static Workspace g_ws[kMaxDevices];
+// Split-K workspaces, one per (device, stream).  Launches on one stream run in order and may share
+// their partials and arrival counters; launches on different streams may overlap and must not.
+static std::map<hipStream_t, Workspace> g_ws[kMaxDevices];
+static size_t g_ws_bytes[kMaxDevices];   // device memory held by the workspaces of a device (retired buffers included)
 static DeviceInfo g_dev[kMaxDevices];
 static bool g_dev_known[kMaxDevices];
 
@@ -65,27 +71,71 @@ int get_device_info(DeviceInfo** out) {
     return g_dev[dev].is_gfx950 ? SG_SUCCESS : SG_NO_DEVICE;
 }
 
-int get_workspace(Workspace** out) {
+static size_t round_up_pow2(size_t v, size_t floor) {
+    size_t r = floor;
+    while (r < v) r <<= 1;
+    return r;
+}
+
+// Device memory for a workspace.  A stream under capture in the default (global) capture mode refuses
+// allocation calls made by its thread; the mode is relaxed for the duration of the call, which
+// records nothing into the graph.
+static void* workspace_alloc(size_t bytes) {
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        p = nullptr;
+    }
+    if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode);
+    return p;
+}
+
+__global__ void fill_zero_kernel(unsigned* p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+// Zeroes n words on `stream` with a kernel (not a memset: a memset node recorded into a captured
+// graph is not reliable on replays), so that every later launch on that stream finds them zero.
+static int fill_zero(unsigned* p, size_t n, hipStream_t stream) {
+    const unsigned grid = (unsigned)((n + 255) / 256 < 1024 ? (n + 255) / 256 : 1024);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, stream, p, n);
+    if (report_hip("fill_zero_kernel", hipGetLastError()) != hipSuccess) return SG_LAUNCH_FAILED;
+    return SG_SUCCESS;
+}
+
+// The workspace of `stream` on the current device, grown to hold partial_bytes of fp32 partials and
+// n_counters arrival counters.  A buffer that is outgrown is kept until the process ends (launches
+// already enqueued may still use it); sizes double, so what is kept is less than what is in use.
+int get_workspace(hipStream_t stream, size_t partial_bytes, size_t n_counters, Workspace* out) {
+    if (partial_bytes > kMaxPartialBytes || n_counters > kMaxCounters) return SG_WORKSPACE_TOO_SMALL;
     int dev;
     if (int rc = current_device(&dev)) return rc;
     std::lock_guard<std::mutex> lock(g_mutex);
-    Workspace& w = g_ws[dev];
-    if (!w.partials) {
-        void* p = nullptr;
-        void* c = nullptr;
-        if (hipMalloc(&p, kPartialBytes) != hipSuccess || hipMalloc(&c, kCounters * sizeof(unsigned)) != hipSuccess ||
-            hipMemset(c, 0, kCounters * sizeof(unsigned)) != hipSuccess) {
-            (void)hipGetLastError();
-            if (p) (void)hipFree(p);
-            if (c) (void)hipFree(c);
-            return SG_NO_DEVICE;
-        }
+    Workspace& w = g_ws[dev][stream];
+    if (w.partial_bytes < partial_bytes) {
+        const size_t bytes = round_up_pow2(partial_bytes, kMinPartialBytes);
+        void* p = workspace_alloc(bytes);
+        if (!p) return SG_NO_DEVICE;
         w.partials = static_cast<float*>(p);
-        w.counters = static_cast<unsigned*>(c);
-        w.partial_bytes = kPartialBytes;
-        w.n_counters = kCounters;
+        w.partial_bytes = bytes;
+        g_ws_bytes[dev] += bytes;
     }
-    *out = &w;
+    if (w.n_counters < n_counters) {
+        const size_t n = round_up_pow2(n_counters, kMinCounters);
+        void* c = workspace_alloc(n * sizeof(unsigned));
+        if (!c) return SG_NO_DEVICE;
+        // in stream order before the launch that asked for them (and every later one on this stream)
+        if (int rc = fill_zero(static_cast<unsigned*>(c), n, stream)) {
+            (void)hipFree(c);
+            return rc;
+        }
+        w.counters = static_cast<unsigned*>(c);
+        w.n_counters = n;
+        g_ws_bytes[dev] += n * sizeof(unsigned);
+    }
+    *out = w;
     return SG_SUCCESS;
 }
 
@@ -103,12 +153,32 @@ struct Config {
     int split_k;  // workgroups per tile, splitting K among themselves
     int nt;       // weights loaded with the non-temporal hint
     int persist;  // LDS engine: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU walking the tiles
+    const Workspace* fixed_ws = nullptr;   // split-K partials and counters to use instead of the stream's own workspace
     int wavetile; // LDS engine, bits 0-1: 1 = every wave owns whole tiles, activations resident in LDS (persist = workgroups per CU);
                   //             2 = persistent K-split workgroups with the activations resident in LDS
                   //             3 = ... resident in the waves' registers (k = 256 * waves * {1, 2, 4});  bit 2: epilogue wave
 };
 
-static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out) {
+// Split-K partials (fp32) and arrival counters for `tiles` output tiles of per_tile_bytes each: the caller's
+// fixed workspace if the configuration names one, the launch stream's own otherwise.
+static int attach_workspace(const Config& c, StreamArgs& a, size_t tiles, size_t per_tile_bytes, hipStream_t stream) {
+    a.ws = nullptr;
+    a.counters = nullptr;
+    if (c.split_k <= 1) return SG_SUCCESS;
+    const size_t need = tiles * c.split_k * per_tile_bytes;
+    Workspace w;
+    if (c.fixed_ws) {
+        w = *c.fixed_ws;
+        if (tiles > w.n_counters || need > w.partial_bytes) return SG_WORKSPACE_TOO_SMALL;
+    } else if (int rc = get_workspace(stream, need, tiles, &w)) {
+        return rc;
+    }
+    a.ws = w.partials;
+    a.counters = w.counters;
+    return SG_SUCCESS;
+}
+
+static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out, hipStream_t stream) {
     const int frags = c.rg * c.mt;
     if (c.waves < 1 || c.waves > 16 || c.depth < 1 || c.rg < 1 || c.mt < 1 || stage_bytes_k < 16) return SG_INVALID_CONFIG;
     a.waves = c.waves;
@@ -119,22 +189,14 @@ static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* ti
     if (c.split_k < 1 || c.split_k > total_stages) return SG_INVALID_CONFIG;
     const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
     if (tiles * c.split_k > 0x7fffffffu) return SG_BAD_ARGUMENT;
-    a.ws = nullptr;
-    a.counters = nullptr;
-    if (c.split_k > 1) {
-        Workspace* w;
-        if (int rc = get_workspace(&w)) return rc;
-        if (tiles > w->n_counters || tiles * c.split_k * frags * 1024 > w->partial_bytes) return SG_WORKSPACE_TOO_SMALL;
-        a.ws = w->partials;
-        a.counters = w->counters;
-    }
+    if (int rc = attach_workspace(c, a, tiles, (size_t)frags * 1024, stream)) return rc;
     *tiles_out = tiles;
     return SG_SUCCESS;
 }
 
 static int launch_stream(const Config& c, StreamArgs a, hipStream_t stream) {
     size_t tiles;
-    if (int rc = prepare(c, a, c.ku * 64, &tiles)) return rc;
+    if (int rc = prepare(c, a, c.ku * 64, &tiles, stream)) return rc;
     const size_t lds = c.waves > 1 ? (size_t)c.waves * c.rg * c.mt * 1024 : 0;
     if (lds > 64 * 1024) return SG_INVALID_CONFIG;
     const unsigned grid = (unsigned)(tiles * c.split_k);
@@ -149,7 +211,7 @@ static int launch_stream(const Config& c, StreamArgs a, hipStream_t stream) {
 static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     if (a.k % 256 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     size_t tiles;
-    if (int rc = prepare(c, a, 256, &tiles)) return rc;
+    if (int rc = prepare(c, a, 256, &tiles, stream)) return rc;
     // activation DMA instructions per stage: 4 rows each, rounded up to a compiled count
     int xu = 8;
     if (c.mt == 1) {
@@ -278,16 +340,8 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
     if (c.split_k < 1 || c.split_k > blocks) return SG_INVALID_CONFIG;
     const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
     if (tiles * c.split_k > 0x7fffffffu) return SG_BAD_ARGUMENT;
-    a.ws = nullptr;
-    a.counters = nullptr;
-    if (c.split_k > 1) {
-        Workspace* w;
-        if (int rc = get_workspace(&w)) return rc;
-        const size_t per_tile = (size_t)c.waves * c.rg * c.mt * 1024;   // fp32 fragments of one workgroup tile
-        if (tiles > w->n_counters || tiles * c.split_k * per_tile > w->partial_bytes) return SG_WORKSPACE_TOO_SMALL;
-        a.ws = w->partials;
-        a.counters = w->counters;
-    }
+    // fp32 fragments of one workgroup tile
+    if (int rc = attach_workspace(c, a, tiles, (size_t)c.waves * c.rg * c.mt * 1024, stream)) return rc;
     // c.ku: ring slots of the activations (0 or out of range = as many as the weights')
     const int dx = (c.ku >= 2 && c.ku < c.depth) ? c.ku : c.depth;
     const size_t lds = ((size_t)c.depth * bn + (size_t)dx * bm) * 128 + (c.split_k > 1 ? 16 : 0);
@@ -380,7 +434,7 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
 static int launch_sparse_engine(const Config& c, StreamArgs a, const uint8_t* meta, hipStream_t stream) {
     if (a.k % 512 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     size_t tiles;
-    if (int rc = prepare(c, a, 512, &tiles)) return rc;
+    if (int rc = prepare(c, a, 512, &tiles, stream)) return rc;
     int xu2 = 16;
     if (c.mt == 1) {
         const int need = (a.m + 3) / 4;
@@ -462,6 +516,33 @@ static int check_pointers(const void* A, const void* B, const void* D, int m, in
     return SG_SUCCESS;
 }
 
+// Register-streaming engine: any k that is a multiple of 16.
+static Config direct_config(int m, int n, int k, int cu_count) {
+    Config c;
+    c.mt = m <= 16 ? 1 : 2;
+    c.nt = 1;
+    c.split_k = 1;
+    c.persist = 0;
+    c.wavetile = 0;
+    const int tiles16 = (n + 15) / 16;
+    c.engine = ENGINE_DIRECT;
+    c.ku = (k % 256 == 0) ? 4 : ((k % 128 == 0) ? 2 : 1);
+    const int stages = (k + c.ku * 64 - 1) / (c.ku * 64);
+    c.rg = tiles16 >= 8 * cu_count ? 2 : 1;
+    const int n_tiles = (n + 16 * c.rg - 1) / (16 * c.rg);
+    const int m_tiles = (m + 16 * c.mt - 1) / (16 * c.mt);
+    c.waves = stages >= 16 ? 8 : (stages >= 4 ? 4 : (stages >= 2 ? 2 : 1));
+    // few tiles: spread K over more workgroups until half the CUs have one
+    while ((long)n_tiles * m_tiles * c.split_k < cu_count / 2 && stages / (c.split_k * 2) >= 2 * c.waves &&
+           c.split_k < 16)
+        c.split_k *= 2;
+    const int per_wave = stages / (c.split_k * c.waves);
+    c.depth = per_wave >= 4 ? 4 : (per_wave >= 2 ? 2 : 1);
+    while (stream_regs(c.mt, c.rg, c.ku, c.depth) > 128 && c.depth > 1) c.depth--;
+    if (c.depth == 3 && c.ku == 8) c.depth = 2;
+    return c;
+}
+
 // Shape -> configuration.  Weights are streamed once, so the only goals are (1) enough
 // loads in flight on every CU to cover HBM latency and (2) long contiguous runs per weight
 // row.  The LDS ring wins wherever it applies (k a multiple of 256); the register-streaming
@@ -541,22 +622,7 @@ static Config pick_config(int m, int n, int k, int cu_count) {
         if (c.depth == 5 || c.depth == 7) c.depth--;
         return c;
     }
-    c.engine = ENGINE_DIRECT;
-    c.ku = (k % 256 == 0) ? 4 : ((k % 128 == 0) ? 2 : 1);
-    const int stages = (k + c.ku * 64 - 1) / (c.ku * 64);
-    c.rg = tiles16 >= 8 * cu_count ? 2 : 1;
-    const int n_tiles = (n + 16 * c.rg - 1) / (16 * c.rg);
-    const int m_tiles = (m + 16 * c.mt - 1) / (16 * c.mt);
-    c.waves = stages >= 16 ? 8 : (stages >= 4 ? 4 : (stages >= 2 ? 2 : 1));
-    // few tiles: spread K over more workgroups until half the CUs have one
-    while ((long)n_tiles * m_tiles * c.split_k < cu_count / 2 && stages / (c.split_k * 2) >= 2 * c.waves &&
-           c.split_k < 16)
-        c.split_k *= 2;
-    const int per_wave = stages / (c.split_k * c.waves);
-    c.depth = per_wave >= 4 ? 4 : (per_wave >= 2 ? 2 : 1);
-    while (stream_regs(c.mt, c.rg, c.ku, c.depth) > 128 && c.depth > 1) c.depth--;
-    if (c.depth == 3 && c.ku == 8) c.depth = 2;
-    return c;
+    return direct_config(m, n, k, cu_count);
 }
 
 static Config config_from_tuning(const SgTuning& t) {
@@ -601,17 +667,34 @@ static bool rejected_before_launch(int rc) {
            rc == SG_WORKSPACE_TOO_SMALL;
 }
 
-// The table's record for the shape if it has a usable one, the heuristics' otherwise.
-static int launch_chosen(const StreamArgs& a, int cu_count, hipStream_t stream) {
+// The table's record for the shape if it has a usable one, the heuristics' otherwise.  Should a launch
+// function refuse the heuristics' own record before anything is enqueued (split-K partials beyond the
+// workspace limit, a combination nothing is compiled for), the same record without the K split and then
+// the register-streaming engine, which takes every legal shape, are tried.
+static int launch_chosen(const StreamArgs& a, int cu_count, hipStream_t stream, const Workspace* fixed_ws = nullptr) {
     SgTuning t;
     if (table_lookup(a.m, a.n, a.k, &t) && t.engine != ENGINE_AUTO) {
-        const Config c = config_from_tuning(t);
+        Config c = config_from_tuning(t);
+        c.fixed_ws = fixed_ws;
         if (c.engine == ENGINE_MID || c.mt == 1 || c.mt == 2) {
             const int rc = launch_config(c, a, stream);
             if (!rejected_before_launch(rc)) return rc;
         }
     }
-    return launch_config(heuristic_config(a.m, a.n, a.k, cu_count), a, stream);
+    Config c = heuristic_config(a.m, a.n, a.k, cu_count);
+    c.fixed_ws = fixed_ws;
+    int rc = launch_config(c, a, stream);
+    if (rejected_before_launch(rc) && c.split_k > 1) {
+        c.split_k = 1;
+        rc = launch_config(c, a, stream);
+    }
+    if (rejected_before_launch(rc)) {
+        c = direct_config(a.m, a.n, a.k, cu_count);
+        c.fixed_ws = fixed_ws;
+        c.split_k = 1;
+        rc = launch_config(c, a, stream);
+    }
+    return rc;
 }
 
 }  // namespace sg
@@ -638,14 +721,21 @@ const char* sg_strerror(int code) {
     }
 }
 
-int sg_init(void) {
+int sg_init(void) { return sg_init_stream(nullptr, kDefaultPartialBytes); }
+
+int sg_init_stream(void* stream, size_t partial_bytes) {
     DeviceInfo* d;
     if (int rc = get_device_info(&d)) return rc;
-    Workspace* w;
-    return get_workspace(&w);
+    Workspace w;
+    return get_workspace(static_cast<hipStream_t>(stream), partial_bytes, kMinCounters, &w);
 }
 
-size_t sg_workspace_bytes(void) { return kPartialBytes + kCounters * sizeof(unsigned); }
+size_t sg_workspace_bytes(void) {
+    int dev;
+    if (current_device(&dev)) return 0;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    return g_ws_bytes[dev];
+}
 
 int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,
                    int b_stride, int split_k, int A_producers, int B_producers, int consumers, int b_lanes, int qsize,

@@ -77,14 +77,15 @@ inline int request_dynamic_lds(const void* kernel, size_t lds, LdsGranted& grant
     return SG_SUCCESS;
 }
 
-// Split-K workspace of the current device (created on first use).
+// Split-K workspace: fp32 partial fragments and one arrival counter per output tile.
 struct Workspace {
     float* partials = nullptr;
     unsigned* counters = nullptr;
     size_t partial_bytes = 0;
     size_t n_counters = 0;
 };
-int get_workspace(Workspace** out);
+// The workspace of `stream` on the current device, created or grown on demand; *out is a copy.
+int get_workspace(hipStream_t stream, size_t partial_bytes, size_t n_counters, Workspace* out);
 
 // Device facts queried once per device.
 struct DeviceInfo {

@@ -41,11 +41,11 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) {
 // 64 lanes x 16 bytes from global memory to LDS [lds_base + 16*lane]; lds_base is wave-uniform.
 __device__ __forceinline__ void dma_1kb(const void* gptr, unsigned lds_base) {
     lds_base = __builtin_amdgcn_readfirstlane(lds_base);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_base) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_base) : "memory", "m0");
 }
 __device__ __forceinline__ void dma_1kb_stream(const void* gptr, unsigned lds_base) {
     lds_base = __builtin_amdgcn_readfirstlane(lds_base);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_base) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_base) : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {

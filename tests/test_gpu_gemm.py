@@ -521,10 +521,15 @@ def test_nan_codes_poison_exactly_their_row_and_column(sg, oracle, m, n, k):
 
 def test_concurrent_launches_from_threads_on_their_own_streams(sg, oracle):
     """The launchers keep no per-call state (skinny_gemm_caller.cu: enqueue on the given stream and return), so host
-    threads may launch at the same time on different streams; split-K shapes are left out because their workspace is
-    one per device.  Every thread's results must equal the ones computed alone, bit for bit."""
+    threads may launch at the same time on different streams.  That includes shapes for which the library splits K on
+    its own (32 x 4096 x 14336, 64 x 8192 x 8192, a short and wide direct-engine shape): split-K workspaces are per
+    stream.  Every thread's results must equal the ones computed alone, bit for bit."""
     import threading
-    shapes = [(8, 4096, 4096), (32, 6144, 1024), (128, 1024, 2048), (16, 2000, 528)]
+    shapes = [(8, 4096, 4096), (32, 6144, 1024), (128, 1024, 2048), (16, 2000, 528), (32, 4096, 14336),
+              (64, 8192, 8192), (8, 64, 16400)]
+    for m, n, k in shapes[4:]:
+        t, _ = sg.skinny_gemm_choice(m, n, k)
+        assert t.split_k > 1, "the heuristics no longer split (%d, %d, %d): pick another shape" % (m, n, k)
     work = []
     for i, (m, n, k) in enumerate(shapes):
         a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=30 + i)
