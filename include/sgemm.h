@@ -146,6 +146,17 @@ typedef struct SgTuning {
 int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
                          int m, int n, int k, int b_stride, const SgTuning* tuning, void* stream);
 
+/* sg_skinny_gemm_tuned for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  No counterpart in the reference.  Same arguments, same kernels,
+ * same result bits; the split-K partials and arrival counters live in a fixed array inside the library's
+ * device image (8 MB + 4096 counters per GPU, held until the process ends) instead of a workspace from
+ * hipMalloc, and nothing is allocated or freed by the call.  A configuration whose partials need more
+ * (tiles * split_k * fragment bytes > 8 MB, or more than 4096 output tiles with split_k > 1) is refused
+ * with SG_WORKSPACE_TOO_SMALL; without a K split there is no limit.  All calls on one GPU share the array:
+ * calls that overlap on one GPU (two streams, unordered graph nodes) race, calls in stream order do not. */
+int sg_skinny_gemm_tuned_noalloc(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                                 int m, int n, int k, int b_stride, const SgTuning* tuning, void* stream);
+
 /* The configuration sg_skinny_gemm_auto would use, for logging and tuning drivers.
  * out[8] = {split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops}. */
 int sg_skinny_gemm_pick(int m, int n, int k, int out[8]);

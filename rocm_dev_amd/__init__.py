@@ -21,6 +21,7 @@ from .api import (  # noqa: F401
     skinny_gemm_pick,
     skinny_gemm_rowcol,
     skinny_gemm_tuned,
+    skinny_gemm_tuned_noalloc,
     init_stream,
     workspace_bytes,
     strerror,

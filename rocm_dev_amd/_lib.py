@@ -26,6 +26,7 @@ SIGNATURES = {
     "sg_skinny_gemm_auto": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm_rowcol": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm_tuned": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "sg_skinny_gemm_tuned_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sg_skinny_gemm_pick": (_i, [_i, _i, _i, C.POINTER(_i * 8)]),
     "sg_skinny_gemm_choice": (_i, [_i, _i, _i, _vp, C.POINTER(_i)]),
     "sg_tuning_set": (_i, [_i, _i, _i, _vp]),

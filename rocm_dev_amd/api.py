@@ -135,6 +135,22 @@ def skinny_gemm_tuned(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k=1, wave
     return _done(rc, check)
 
 
+def skinny_gemm_tuned_noalloc(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k=1, waves=4, row_tiles=1, m_blocks=None,
+                              depth=2, k_chunks=4, non_temporal=1, persistent_wgs_per_cu=0, wave_tiles=0, check=False):
+    """skinny_gemm_tuned with the split-K partials in the library's fixed device array: allocates nothing, refuses
+    configurations whose partials exceed 8 MB or 4096 tiles with WORKSPACE_TOO_SMALL (no reference counterpart)."""
+    m, k = A.shape
+    n = B.shape[0]
+    if m_blocks is None:
+        m_blocks = 1 if m <= 16 else 2
+    t = SgTuning(engine, split_k, waves, row_tiles, m_blocks, depth, k_chunks, non_temporal, persistent_wgs_per_cu, wave_tiles)
+    with torch.cuda.device(A.device):
+        rc = lib.sg_skinny_gemm_tuned_noalloc(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
+                                              _dev(scale_tensor, torch.float32), m, n, k, B.stride(0), C.byref(t),
+                                              _stream())
+    return _done(rc, check)
+
+
 def init_stream(stream=None, partial_bytes=64 << 20, check=True):
     """Create the split-K workspace of `stream` (torch stream; None = torch's current stream) ahead of time."""
     handle = _stream() if stream is None else stream.cuda_stream

@@ -139,6 +139,34 @@ int get_workspace(hipStream_t stream, size_t partial_bytes, size_t n_counters, W
     return SG_SUCCESS;
 }
 
+// ---- scratch for the entry point that allocates nothing -------------------------------------------
+// Split-K partials and arrival counters of sg_skinny_gemm_tuned_noalloc live in this array instead of a
+// workspace from hipMalloc.  Every device the library runs on holds its own copy at its own address; in host
+// code the name below is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t kStaticPartialBytes = 8u << 20;
+constexpr size_t kStaticCounters = 4096;
+static __device__ __align__(256) unsigned char scratch[kStaticPartialBytes + kStaticCounters * sizeof(unsigned)];
+static unsigned char* g_scratch_ptr[kMaxDevices];   // device address of `scratch` per device, looked up once
+
+static int static_workspace(Workspace* out) {
+    int dev;
+    if (int rc = current_device(&dev)) return rc;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        if (report_hip("hipGetSymbolAddress", hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            return SG_NO_DEVICE;
+        }
+        g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+    }
+    out->partials = reinterpret_cast<float*>(g_scratch_ptr[dev]);
+    out->partial_bytes = kStaticPartialBytes;
+    out->counters = reinterpret_cast<unsigned*>(g_scratch_ptr[dev] + kStaticPartialBytes);
+    out->n_counters = kStaticCounters;
+    return SG_SUCCESS;
+}
+
 // ---- kernel dispatch ------------------------------------------------------------------------
 enum Engine { ENGINE_AUTO = 0, ENGINE_DIRECT = 1, ENGINE_LDS = 2, ENGINE_RING = 3, ENGINE_MID = 4 };
 
@@ -815,6 +843,33 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D, const floa
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
     a.out_f32 = 0;
+    return launch_config(c, a, static_cast<hipStream_t>(stream));
+}
+
+int sg_skinny_gemm_tuned_noalloc(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n,
+                                 int k, int b_stride, const SgTuning* t, void* stream) {
+    if (!t) return SG_BAD_ARGUMENT;
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 16 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (int rc = check_pointers(A, B, D, m, n, k, b_stride)) return rc;
+    if (!scale_tensor) return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    Workspace w;
+    if (int rc = static_workspace(&w)) return rc;
+    Config c = config_from_tuning(*t);
+    if (c.engine == ENGINE_AUTO) c = heuristic_config(m, n, k, dev->cu_count);
+    if (c.engine != ENGINE_MID && c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
+    c.fixed_ws = &w;
+    StreamArgs a{};
+    a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
+    a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
+    a.out_f32 = 0;
+    // The array keeps whatever the last call left.  The partials are written before they are read; the arrival
+    // counters must start at zero, and although a launch that completes leaves them at zero they are cleared
+    // here, in stream order, with a kernel (a memset node would not be safe in a captured graph).
+    if (c.split_k > 1)
+        if (int rc = fill_zero(w.counters, w.n_counters, static_cast<hipStream_t>(stream))) return rc;
     return launch_config(c, a, static_cast<hipStream_t>(stream));
 }
 

@@ -1,0 +1,74 @@
+"""sg_skinny_gemm_tuned_noalloc: the entry point that allocates nothing must reproduce sg_skinny_gemm_tuned bit for bit.
+
+Its split-K partials and arrival counters live in a fixed array of the library's device image that every call on the
+GPU shares and that keeps the last call's contents, so the check is made on two calls in a row, the second on a
+smaller problem, and both against the existing entry point and the CPU oracle.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import GEMM_TOL, bits, dev, scale_tensor
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def sg():
+    import rocm_dev_amd
+    return rocm_dev_amd
+
+
+# (m, n, k, tuning): LDS ring with a 4-way and a 2-way K split, the register-streaming engine split 4 ways, the
+# mid-batch engine split 2 ways, and the library's own choice for a shape where it splits K itself
+CASES = [
+    [(32, 4096, 14336, dict(engine=2, split_k=4, waves=2, row_tiles=2, m_blocks=2, depth=3)),
+     (8, 1024, 4096, dict(engine=2, split_k=2, waves=2, row_tiles=1, m_blocks=1, depth=4))],
+    [(16, 2048, 8192 + 64, dict(engine=1, split_k=4, waves=4, row_tiles=1, m_blocks=1, depth=2, k_chunks=1)),
+     (5, 130, 1040, dict(engine=1, split_k=2, waves=2, row_tiles=1, m_blocks=1, depth=2, k_chunks=1))],
+    [(128, 2048, 8192, dict(engine=4, split_k=2, waves=8, row_tiles=2, m_blocks=2, depth=3, k_chunks=0)),
+     (64, 512, 4096, dict(engine=4, split_k=2, waves=4, row_tiles=2, m_blocks=2, depth=2, k_chunks=0))],
+    [(32, 4096, 14336, dict(engine=0)),
+     (32, 1024, 14336, dict(engine=0))],
+]
+
+
+@pytest.mark.parametrize("pair", CASES)
+def test_noalloc_matches_tuned_on_two_calls_in_a_row(sg, oracle, pair):
+    for call, (m, n, k, tuning) in enumerate(pair):
+        a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=70 + call)
+        A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+        want = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        print("case", call, m, n, k, tuning, flush=True)
+        assert sg.skinny_gemm_tuned(A, B, want, S, **tuning) == 0
+        before = torch.cuda.memory_allocated(), sg.workspace_bytes()
+        rc = sg.skinny_gemm_tuned_noalloc(A, B, got, S, **tuning)
+        assert rc == 0, sg.strerror(rc)
+        torch.cuda.synchronize()
+        assert (torch.cuda.memory_allocated(), sg.workspace_bytes()) == before
+        assert np.array_equal(bits(got), bits(want)), "differs from sg_skinny_gemm_tuned"
+        if m * n * k <= 32 * 4096 * 14336:
+            ref = oracle.gemm_omp(a8, b8, scale)
+            assert oracle.max_rel_err_bf16(bits(got), ref) <= GEMM_TOL
+
+
+def test_noalloc_refuses_partials_beyond_its_array(sg, oracle):
+    """8 MB of partials, 4096 counters: a 4-way split of 256 x 8192 tiles of 128 x 128 needs 64 * 2 * 4 * 64 KB."""
+    m, n, k = 256, 8192, 8192
+    A = torch.zeros((m, k), dtype=torch.uint8, device="cuda")
+    B = torch.zeros((n, k), dtype=torch.uint8, device="cuda")
+    D = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    S = scale_tensor(1.0)
+    rc = sg.skinny_gemm_tuned_noalloc(A, B, D, S, engine=4, split_k=4, waves=8, row_tiles=2, m_blocks=4, depth=3, k_chunks=0)
+    assert rc == sg.SgReturnCode.WORKSPACE_TOO_SMALL
+    # more than 4096 output tiles with a K split
+    B2 = torch.zeros((16 * 4097, 512), dtype=torch.uint8, device="cuda")
+    A2 = torch.zeros((8, 512), dtype=torch.uint8, device="cuda")
+    D2 = torch.zeros((8, 16 * 4097), dtype=torch.bfloat16, device="cuda")
+    rc = sg.skinny_gemm_tuned_noalloc(A2, B2, D2, S, engine=2, split_k=2, waves=1, row_tiles=1, m_blocks=1, depth=1)
+    assert rc == sg.SgReturnCode.WORKSPACE_TOO_SMALL
+    # without a K split nothing is needed from the array
+    rc = sg.skinny_gemm_tuned_noalloc(A2, B2, D2, S, engine=2, split_k=1, waves=1, row_tiles=1, m_blocks=1, depth=2)
+    torch.cuda.synchronize()
+    assert rc == 0
