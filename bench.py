@@ -64,6 +64,10 @@ def main():
                          "on cold weights through the library's choice and three times through the one-wave-workgroup kernel "
                          "it replaced, after three 256 MiB copies of known traffic, and exit (for L2 / HBM traffic counter runs; "
                          "prints no JSON line)")
+    ap.add_argument("--stamps", action="store_true",
+                    help="only run the decode GEMMs (four projection shapes at M = --m) back to back from a HIP graph with "
+                         "the library's per-workgroup time stamps switched on, and print where a launch period goes "
+                         "(launch gap, prologue, first data, streaming, epilogue); prints no JSON line")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1")
@@ -78,6 +82,68 @@ def main():
     torch.manual_seed(0)
     if lib.sg_init() != 0:
         sys.exit("bench.py: sg_init failed")
+
+    if args.stamps:
+        import numpy as np
+        one = torch.ones(1, device="cuda")
+        reps = 24
+        print("in-kernel time stamps, M = %d, graph of %d back-to-back launches on cold weights, medians over launches 4..%d"
+              % (args.m, reps, reps - 1))
+        print("all times in us; gap = first entry of a launch - last end of the one before; spread = last - first entry")
+        side = torch.cuda.Stream()
+        for name, (n, k) in SHAPES.items():
+            copies = max(3, int(COLD_BYTES // (n * k)) + 1)
+            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(copies)]
+            a8 = torch.randint(0, 0x7E, (args.m, k), device="cuda", dtype=torch.uint8)
+            d = torch.empty((args.m, n), device="cuda", dtype=torch.bfloat16)
+            words = reps * 4096 * 8
+            buf = torch.zeros(words, device="cuda", dtype=torch.int64)
+            torch.cuda.synchronize()
+            lib.sg_debug_stamps(buf.data_ptr(), words)
+            with torch.cuda.stream(side):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    st = torch.cuda.current_stream().cuda_stream
+                    for i in range(reps):
+                        rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(),
+                                                     args.m, n, k, k, st)
+                        if rc != 0:
+                            raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
+                lib.sg_debug_stamps(None, 0)
+                ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                for _ in range(20):
+                    g.replay()
+                ev0.record()
+                g.replay()
+                ev1.record()
+                torch.cuda.synchronize()
+            period_ev = ev0.elapsed_time(ev1) * 1e3 / reps
+            raw = buf.cpu().numpy().astype(np.uint64).reshape(-1, 8)
+            used = int(np.count_nonzero(raw[:, 0]))
+            grid = used // reps
+            t = raw[:used].reshape(reps, grid, 8)
+            tick = 0.01   # 100 MHz constant clock
+            ent, iss, land, cons, end = (t[:, :, i].astype(np.int64) * tick for i in range(5))
+            rows = []
+            for j in range(4, reps):
+                e0 = ent[j].min()
+                rows.append({
+                    "gap": e0 - end[j - 1].max(), "period": e0 - ent[j - 1].min(), "spread": ent[j].max() - e0,
+                    "issue": np.median(iss[j] - ent[j]), "land_med": np.median(land[j] - ent[j]),
+                    "land_max": (land[j] - ent[j]).max(), "stream": np.median(cons[j] - land[j]),
+                    "epi": np.median(end[j] - cons[j]), "wg_med": np.median(end[j] - ent[j]), "wg_max": (end[j] - ent[j]).max(),
+                    "span": end[j].max() - e0, "tail": end[j].max() - np.median(end[j]),
+                    "mhz": np.median((t[j, :, 6].astype(np.int64) - t[j, :, 5].astype(np.int64)) / np.maximum(end[j] - ent[j], tick))})
+            med = {key: float(np.median([r[key] for r in rows])) for key in rows[0]}
+            t_choice, _ = sg.skinny_gemm_choice(args.m, n, k)
+            print("%-8s %5d x %5d  grid %4d  event-pair period %.2f | period %.2f = gap %.2f + span %.2f | entry spread %.2f | "
+                  "workgroup (median): prologue issue %.2f, first stage landed %.2f (max %.2f), streaming %.2f, reduce+store %.2f, "
+                  "total %.2f (max %.2f) | last end - median end %.2f | shader clock %.0f MHz | %s"
+                  % (name, n, k, grid, period_ev, med["period"], med["gap"], med["span"], med["spread"], med["issue"], med["land_med"],
+                     med["land_max"], med["stream"], med["epi"], med["wg_med"], med["wg_max"], med["tail"], med["mhz"],
+                     sg.api.tuning_as_dict(t_choice)), flush=True)
+            del wb, buf
+        return
 
     if args.decode_counters:
         one = torch.ones(1, device="cuda")

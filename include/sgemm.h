@@ -186,6 +186,15 @@ int sg_tuning_clear(void);
 int sg_tuning_load(const char* path);
 int sg_tuning_save(const char* path);
 
+/* Profiling aid, no counterpart in the reference.  While a buffer is set, every launch of the LDS-ring GEMM
+ * kernels (per-tile and persistent) takes the next grid * 8 words of it and each workgroup leaves eight 64-bit
+ * words there when it is done: [0] kernel entry, [1] prologue DMAs issued, [2] first stage landed, [3] last stage
+ * consumed, [4] outputs stored and acknowledged - 10 ns ticks of the device's constant 100 MHz clock -
+ * [5], [6] shader clock at entry and end, [7] XCC_ID << 32 | HW_ID.  Launches that no longer fit leave nothing.
+ * A launch recorded into a HIP graph keeps its slice on every replay.  Process-wide; set it from one thread while
+ * no other thread launches.  sg_debug_stamps(NULL, 0) switches the stamps off again. */
+int sg_debug_stamps(unsigned long long* device_buffer, size_t n_words);
+
 /* Replaces  template<class out> void async_gemm(const fp8* A, const fp8* B, out* D, int m,
  * int n, int k)  (async_gemm_sparse/sparse_k.cu:45-69, async_gemm_blanes/sparse_k.cu,
  * async_gemm_16x16x64/src.cu:55-82): D = A * B^T without a scale, default stream, through

@@ -167,6 +167,20 @@ static int static_workspace(Workspace* out) {
     return SG_SUCCESS;
 }
 
+// ---- time stamps (profiling aid) -------------------------------------------------------------------
+static unsigned long long* g_stamp_buf = nullptr;
+static size_t g_stamp_words = 0, g_stamp_cursor = 0;
+
+// Room for one launch of `grid` workgroups, or nullptr when stamps are off or the buffer is full.
+static unsigned long long* take_stamps(unsigned grid) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    const size_t need = (size_t)grid * kStampWords;
+    if (!g_stamp_buf || g_stamp_cursor + need > g_stamp_words) return nullptr;
+    unsigned long long* p = g_stamp_buf + g_stamp_cursor;
+    g_stamp_cursor += need;
+    return p;
+}
+
 // ---- kernel dispatch ------------------------------------------------------------------------
 enum Engine { ENGINE_AUTO = 0, ENGINE_DIRECT = 1, ENGINE_LDS = 2, ENGINE_RING = 3, ENGINE_MID = 4 };
 
@@ -218,6 +232,7 @@ static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* ti
     const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
     if (tiles * c.split_k > 0x7fffffffu) return SG_BAD_ARGUMENT;
     if (int rc = attach_workspace(c, a, tiles, (size_t)frags * 1024, stream)) return rc;
+    set_reciprocals(a);
     *tiles_out = tiles;
     return SG_SUCCESS;
 }
@@ -295,6 +310,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     if (lds > 159 * 1024) return SG_INVALID_CONFIG;  // 160 KB per CU, minus the kernel's static LDS
     const unsigned threads = (unsigned)(c.waves + extra_wave) * 64;
     if (threads > 1024) return SG_TOO_MANY_WARPS;
+    if (mode == 0 || mode == 1 || mode == 3) a.stamps = take_stamps(grid);
 #define SG_GO(MT, RG)                                                                                          \
     if (c.mt == MT && c.rg == RG)                                                                              \
         return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, mode, a, grid, threads, lds, stream);
@@ -319,6 +335,7 @@ static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
     a.m_tiles = (a.m + 16 * c.mt - 1) / (16 * c.mt);
     a.ws = nullptr;
     a.counters = nullptr;
+    set_reciprocals(a);
     const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
     if (tiles > 0x7fffffffu) return SG_BAD_ARGUMENT;
     int xu = 8;
@@ -370,6 +387,7 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
     if (tiles * c.split_k > 0x7fffffffu) return SG_BAD_ARGUMENT;
     // fp32 fragments of one workgroup tile
     if (int rc = attach_workspace(c, a, tiles, (size_t)c.waves * c.rg * c.mt * 1024, stream)) return rc;
+    set_reciprocals(a);
     // c.ku: ring slots of the activations (0 or out of range = as many as the weights')
     const int dx = (c.ku >= 2 && c.ku < c.depth) ? c.ku : c.depth;
     const size_t lds = ((size_t)c.depth * bn + (size_t)dx * bm) * 128 + (c.split_k > 1 ? 16 : 0);
@@ -763,6 +781,14 @@ size_t sg_workspace_bytes(void) {
     if (current_device(&dev)) return 0;
     std::lock_guard<std::mutex> lock(g_mutex);
     return g_ws_bytes[dev];
+}
+
+int sg_debug_stamps(unsigned long long* device_buffer, size_t n_words) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_stamp_buf = n_words ? device_buffer : nullptr;
+    g_stamp_words = device_buffer ? n_words : 0;
+    g_stamp_cursor = 0;
+    return SG_SUCCESS;
 }
 
 int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,

@@ -49,6 +49,19 @@ __device__ __forceinline__ f32x4 mfma_e4m3_16x16x128(const i32x8& a, const i32x8
 }
 
 
+// n / d for a divisor whose reciprocal the host has prepared: inv = floor(2^32 / d) (0xffffffff for d = 1).
+// The product's high word is the quotient or one below it for every 32-bit n, so one correction step makes
+// it exact.  Five scalar instructions where the compiler's general division is about thirty, among them a
+// reciprocal on the vector unit whose result has to travel back to the scalar unit - at the top of a
+// kernel whose one wave per SIMD has nothing else to issue meanwhile.
+__host__ __device__ __forceinline__ unsigned div_reciprocal(unsigned d) {
+    return d <= 1 ? 0xffffffffu : (unsigned)(0x100000000ull / d);
+}
+__device__ __forceinline__ unsigned fast_div(unsigned n, unsigned d, unsigned inv) {
+    const unsigned q = __umulhi(n, inv);
+    return n - q * d >= d ? q + 1 : q;
+}
+
 // Workgroups are dispatched round-robin over the 8 XCDs (workgroup b runs on XCD b % 8), each with its own
 // L2.  A 16-row tile writes only 32 bytes of every output row, so the four tiles that share a 128-byte line of
 // D should pass through the same L2, which then merges them before they reach memory: workgroup b is given

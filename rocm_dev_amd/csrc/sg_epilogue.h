@@ -31,7 +31,69 @@ struct StreamArgs {
     int split_k, waves;
     int n_tiles, m_tiles;
     int out_f32;
+    unsigned inv_n_tiles, inv_split_k, inv_waves;  // div_reciprocal() of n_tiles, split_k, waves (set_reciprocals)
+    unsigned long long* stamps;  // profiling aid, normally nullptr: kStampWords time stamps per workgroup (sg_debug_stamps)
 };
+
+// Time stamps a workgroup leaves when a.stamps is set (wave 0 writes them when it is done):
+//   [0] kernel entry (first instruction)  [1] prologue DMAs issued  [2] first stage landed  [3] last stage consumed
+//   [4] outputs stored and acknowledged   - all five from the 100 MHz constant clock (10 ns units) -
+//   [5] shader clock at entry  [6] shader clock at the end  [7] hardware id: XCC_ID << 32 | HW_ID
+// The clock reads are unconditional (one scalar instruction each); only the final wait and the stores depend on
+// a.stamps, so a launch without stamps does not wait for that argument before it requests the others.
+constexpr int kStampWords = 8;
+struct Stamps {
+    unsigned long long t[kStampWords];
+    __device__ __forceinline__ void begin() {
+        t[0] = __builtin_amdgcn_s_memrealtime();
+        t[5] = __builtin_amdgcn_s_memtime();
+    }
+    // mark(1) also presets [2] for the paths on which no stage is waited for separately
+    __device__ __forceinline__ void mark(int i) {
+        t[i] = __builtin_amdgcn_s_memrealtime();
+        if (i == 1) t[2] = t[1];
+    }
+    __device__ __forceinline__ void end(const StreamArgs& a) {
+        if (a.stamps == nullptr) return;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        t[4] = __builtin_amdgcn_s_memrealtime();
+        t[6] = __builtin_amdgcn_s_memtime();
+        const unsigned hw = __builtin_amdgcn_s_getreg((31 << 11) | 4), xcc = __builtin_amdgcn_s_getreg((31 << 11) | 20);
+        t[7] = ((unsigned long long)xcc << 32) | hw;
+        if (threadIdx.x == 0) {
+            unsigned long long* out = a.stamps + (size_t)blockIdx.x * kStampWords;
+#pragma unroll
+            for (int i = 0; i < kStampWords; i++) out[i] = t[i];
+        }
+    }
+};
+
+inline void set_reciprocals(StreamArgs& a) {
+    a.inv_n_tiles = div_reciprocal((unsigned)a.n_tiles);
+    a.inv_split_k = div_reciprocal((unsigned)a.split_k);
+    a.inv_waves = div_reciprocal((unsigned)a.waves);
+}
+
+// Position `bid` in tile order -> (tile_n, split, tile_m): n tiles fastest, then the K splits of a tile, then m tiles.
+__device__ __forceinline__ void decode_tile(const StreamArgs& a, int bid, int& tile_n, int& split, int& tile_m) {
+    const unsigned q = fast_div((unsigned)bid, (unsigned)a.n_tiles, a.inv_n_tiles);
+    tile_n = bid - (int)q * a.n_tiles;
+    const unsigned m = fast_div(q, (unsigned)a.split_k, a.inv_split_k);
+    split = (int)(q - m * (unsigned)a.split_k);
+    tile_m = (int)m;
+}
+
+// K range [b_begin, b_end) of split `split` out of `blocks` stage-sized blocks; the last split takes the remainder.
+__device__ __forceinline__ void split_range(const StreamArgs& a, int blocks, int split, int& b_begin, int& b_end) {
+    const int per_split = (int)fast_div((unsigned)blocks, (unsigned)a.split_k, a.inv_split_k);
+    b_begin = split * per_split;
+    b_end = (split == a.split_k - 1) ? blocks : b_begin + per_split;
+}
+
+// Blocks wave `wave` takes when `waves` waves share n_blk blocks round-robin: ceil((n_blk - wave) / waves).
+__device__ __forceinline__ int blocks_of_wave(const StreamArgs& a, int n_blk, int wave) {
+    return wave < n_blk ? (int)fast_div((unsigned)(n_blk - wave + a.waves - 1), (unsigned)a.waves, a.inv_waves) : 0;
+}
 
 // Writes one finished 16(n) x 16(m) fragment: lane owns m = m_base + l%16, n = n_base + 4*(l/16)..+3.
 __device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, float scale, int m_idx, int n_idx) {

@@ -47,6 +47,18 @@ __device__ __forceinline__ void dma_1kb_stream(const void* gptr, unsigned lds_ba
     lds_base = __builtin_amdgcn_readfirstlane(lds_base);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(gptr), "s"(lds_base) : "memory", "m0");
 }
+// The same with the address split into a wave-uniform 64-bit base (scalar registers) and a 32-bit per-lane
+// offset: advancing along K is then one scalar add per stage instead of a 64-bit vector add per instruction.
+__device__ __forceinline__ void dma_1kb_at(const void* sbase, unsigned voff, unsigned lds_base) {
+    lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void dma_1kb_stream_at(const void* sbase, unsigned voff, unsigned lds_base) {
+    lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" ::"v"(voff), "s"(sbase), "s"(lds_base)
+                 : "memory", "m0");
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
@@ -131,45 +143,45 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
     static_assert(XU <= 4 * MT, "more activation rows than the tile has");
 
+    Stamps stamps;
+    stamps.begin();
     const int lane = lane_id();
     const int wave = wave_id();
     const int waves = a.waves;
 
-    int bid = xcd_order((int)blockIdx.x, (int)gridDim.x);
-    const int tile_n = bid % a.n_tiles;
-    bid /= a.n_tiles;
-    const int split = bid % a.split_k;
-    const int tile_m = bid / a.split_k;
+    int tile_n, split, tile_m;
+    decode_tile(a, xcd_order((int)blockIdx.x, (int)gridDim.x), tile_n, split, tile_m);
     const int n0 = tile_n * (16 * RG);
     const int m0 = tile_m * (16 * MT);
 
     // K range of this workgroup in 256-byte blocks; the last split takes the remainder
-    const int blocks = a.k >> 8;
-    const int per_split = blocks / a.split_k;
-    const int b_begin = split * per_split;
-    const int b_end = (split == a.split_k - 1) ? blocks : b_begin + per_split;
-    const int n_blk = b_end - b_begin;
-    const int mine = wave < n_blk ? (n_blk - wave + waves - 1) / waves : 0;
+    int b_begin, b_end;
+    split_range(a, a.k >> 8, split, b_begin, b_end);
+    const int mine = blocks_of_wave(a, b_end - b_begin, wave);
 
-    // ---- DMA source pointers (per lane) ---------------------------------------------------
+    // ---- DMA sources: a wave-uniform base per operand (the tile's first row, advanced along K with scalar
+    // adds) plus a 32-bit offset per lane and instruction (the host keeps 64 rows of either operand below 2 GB)
     const int q = lane >> 2, p = lane & 3;
     const int src_row = q & 3;        // row inside the 4-row instruction
     const int src_kc = q >> 2;        // 64-byte run inside the 256-byte block
-    const uint8_t* wsrc[RG][4];
+    const uint8_t* w_base = a.B + (size_t)n0 * a.b_stride + ((size_t)(b_begin + wave) << 8);
+    const uint8_t* x_base = a.A + (size_t)m0 * a.k + ((size_t)(b_begin + wave) << 8);
+    const int w_last = a.n - 1 - n0, x_last = a.m - 1 - m0;   // rows past the edge re-read the last row, never stored
+    unsigned woff[RG][4];
 #pragma unroll
     for (int rg = 0; rg < RG; rg++)
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            int row = n0 + rg * 16 + 4 * u + src_row;
-            row = row < a.n ? row : a.n - 1;   // past the edge: re-read the last row, never stored
-            wsrc[rg][u] = a.B + (size_t)row * a.b_stride + src_kc * 64 + ((p + u) & 3) * 16;
+            int row = rg * 16 + 4 * u + src_row;
+            row = row < w_last ? row : w_last;
+            woff[rg][u] = (unsigned)row * (unsigned)a.b_stride + src_kc * 64 + ((p + u) & 3) * 16;
         }
-    const uint8_t* xsrc[XU];
+    unsigned xoff[XU];
 #pragma unroll
     for (int u = 0; u < XU; u++) {
-        int row = m0 + 4 * u + src_row;
-        row = row < a.m ? row : a.m - 1;
-        xsrc[u] = a.A + (size_t)row * a.k + src_kc * 64 + ((p + (u & 3)) & 3) * 16;
+        int row = 4 * u + src_row;
+        row = row < x_last ? row : x_last;
+        xoff[u] = (unsigned)row * (unsigned)a.k + src_kc * 64 + ((p + (u & 3)) & 3) * 16;
     }
 
     // ---- LDS read offsets (per lane) ------------------------------------------------------
@@ -178,18 +190,19 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
     const unsigned my_ring_lds = lds_addr(my_ring);
 
+    const size_t k_step = (size_t)waves << 8;
     auto issue = [&](int i) __attribute__((always_inline)) {  // i-th stage of this wave -> slot i % DEPTH
-        const size_t koff = (size_t)(b_begin + wave + i * waves) << 8;
+        const size_t koff = (size_t)i * k_step;
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                if (NT) dma_1kb_stream(wsrc[rg][u] + koff, slot + (rg * 4 + u) * 1024);
-                else dma_1kb(wsrc[rg][u] + koff, slot + (rg * 4 + u) * 1024);
+                if (NT) dma_1kb_stream_at(w_base + koff, woff[rg][u], slot + (rg * 4 + u) * 1024);
+                else dma_1kb_at(w_base + koff, woff[rg][u], slot + (rg * 4 + u) * 1024);
             }
 #pragma unroll
-        for (int u = 0; u < XU; u++) dma_1kb(xsrc[u] + koff, slot + (RG * 4 + u) * 1024);
+        for (int u = 0; u < XU; u++) dma_1kb_at(x_base + koff, xoff[u], slot + (RG * 4 + u) * 1024);
     };
 
     f32x4 acc[RG][MT];
@@ -206,9 +219,11 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     if (mine >= DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) issue(d);
+        stamps.mark(1);
         int i = 0;
         for (; i + DEPTH < mine; i++) {
             wait_vmcnt<(DEPTH - 1) * PER_STAGE>();   // stage i has landed; DEPTH-1 stages still in flight
+            if (i == 0) stamps.mark(2);
             consume(i);
             // the slot is refilled only after its reads have returned: the MFMAs above need the
             // data, and this wait keeps the DMA behind them
@@ -220,14 +235,18 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
         drain_ring<0, DEPTH, PER_STAGE>(consume, i);
     } else {
         for (int i = 0; i < mine; i++) issue(i);
+        stamps.mark(1);
         wait_vmcnt<0>();
+        stamps.mark(2);
         for (int i = 0; i < mine; i++) consume(i);
     }
 
     // the ring is reused for the cross-wave reduction: every wave must be done reading it
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    stamps.mark(3);
     __syncthreads();
     finish_tile<RG, MT>(a, acc, reinterpret_cast<f32x4*>(ring), &arrival, tile_m, tile_n, split, m0, n0);
+    stamps.end(a);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -248,6 +267,8 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     constexpr int FRAGS = RG * MT;
     static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
 
+    Stamps stamps;
+    stamps.begin();
     const int lane = lane_id();
     const int wave = wave_id();
     const int waves = a.waves;
@@ -397,6 +418,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     if (total >= DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) issue(d);
+        stamps.mark(1);
         if (XRES) {
             wait_vmcnt_upto(DEPTH * PER_STAGE);   // this wave's activation blocks are older than its DEPTH stages
             __syncthreads();
@@ -404,6 +426,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
         int i = 0;
         for (; i + DEPTH < total; i++) {
             wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            if (i == 0) stamps.mark(2);
             consume(i);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
@@ -425,6 +448,8 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
             after_consume();
         }
     }
+    stamps.mark(3);   // here the last tile's reduction is part of [3]: the streaming waves run into it
+    stamps.end(a);
 }
 
 // ---------------------------------------------------------------------------------------------

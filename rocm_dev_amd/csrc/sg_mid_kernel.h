@@ -83,18 +83,13 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     const int wn = wave % WN, wm = wave / WN;
     const bool loads_x = XW == WAVES || wave < XW;   // wave-uniform
 
-    int bid = blockIdx.x;
-    const int tile_n = bid % a.n_tiles;
-    bid /= a.n_tiles;
-    const int split = bid % a.split_k;
-    const int tile_m = bid / a.split_k;
+    int tile_n, split, tile_m;
+    decode_tile(a, (int)blockIdx.x, tile_n, split, tile_m);
     const int n0 = tile_n * BN;
     const int m0 = tile_m * BM;
 
-    const int blocks = a.k >> 7;   // 128-byte K blocks
-    const int per_split = blocks / a.split_k;
-    const int b_begin = split * per_split;
-    const int b_end = (split == a.split_k - 1) ? blocks : b_begin + per_split;
+    int b_begin, b_end;
+    split_range(a, a.k >> 7, split, b_begin, b_end);   // 128-byte K blocks
     const int n_blk = b_end - b_begin;
     // Every workgroup walks its K range from a different starting block (and wraps): workgroups that start
     // together would otherwise ask one L2 for the same activation lines at the same moment, block after

@@ -54,20 +54,14 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
     const int wave = wave_id();
     const int waves = a.waves;
 
-    int bid = xcd_order((int)blockIdx.x, (int)gridDim.x);
-    const int tile_n = bid % a.n_tiles;
-    bid /= a.n_tiles;
-    const int split = bid % a.split_k;
-    const int tile_m = bid / a.split_k;
+    int tile_n, split, tile_m;
+    decode_tile(a, xcd_order((int)blockIdx.x, (int)gridDim.x), tile_n, split, tile_m);
     const int n0 = tile_n * (16 * RG);
     const int m0 = tile_m * (16 * MT);
 
-    const int blocks = a.k >> 9;   // 512-k stages
-    const int per_split = blocks / a.split_k;
-    const int b_begin = split * per_split;
-    const int b_end = (split == a.split_k - 1) ? blocks : b_begin + per_split;
-    const int n_blk = b_end - b_begin;
-    const int mine = wave < n_blk ? (n_blk - wave + waves - 1) / waves : 0;
+    int b_begin, b_end;
+    split_range(a, a.k >> 9, split, b_begin, b_end);   // 512-k stages
+    const int mine = blocks_of_wave(a, b_end - b_begin, wave);
 
     // ---- DMA sources ------------------------------------------------------------------------
     const int v_row = lane >> 4, v_pp = lane & 15;     // values / activations: 4 rows x 16 pieces

@@ -94,21 +94,17 @@ stream_gemm_kernel(const StreamArgs a) {
     const int waves = a.waves;
     const int r = lane & 15, g = lane >> 4;
 
-    int bid = xcd_order((int)blockIdx.x, (int)gridDim.x);
-    const int tile_n = bid % a.n_tiles;
-    bid /= a.n_tiles;
-    const int split = bid % a.split_k;
-    const int tile_m = bid / a.split_k;
+    int tile_n, split, tile_m;
+    decode_tile(a, xcd_order((int)blockIdx.x, (int)gridDim.x), tile_n, split, tile_m);
     const int n0 = tile_n * (16 * RG);
     const int m0 = tile_m * (16 * MT);
 
     // K range of this workgroup in stages of STAGE_K bytes; the last split takes the remainder,
     // including a final partial stage when k is not a multiple of STAGE_K
     const int full_stages = a.k / STAGE_K;
-    const int per_split = full_stages / a.split_k;
-    const int s_begin = split * per_split;
+    int s_begin, s_end_full;
+    split_range(a, full_stages, split, s_begin, s_end_full);
     const bool last_split = split == a.split_k - 1;
-    const int s_end_full = last_split ? full_stages : s_begin + per_split;
     const bool has_tail = last_split && (a.k % STAGE_K) != 0;
 
     // Rows past the edge of either operand re-read the last valid row: the MFMA keeps result
@@ -137,7 +133,7 @@ stream_gemm_kernel(const StreamArgs a) {
     // This wave's full stages are  first, first + waves, ...  (mine of them).  The steady-state
     // loop is branch-free so that the compiler can keep DEPTH stages of loads in flight.
     const int n_full = s_end_full - s_begin;
-    const int mine = wave < n_full ? (n_full - wave + waves - 1) / waves : 0;
+    const int mine = blocks_of_wave(a, n_full, wave);
     const int first_off = (s_begin + wave) * STAGE_K;
     const int step_off = waves * STAGE_K;
 

@@ -50,6 +50,7 @@ int skinny_gemm_fastpath(const unsigned char* A, const unsigned char* B, uint16_
     a.n_tiles = (n + 16 * B_LANES_ - 1) / (16 * B_LANES_);
     a.m_tiles = (m + 16 * MT - 1) / (16 * MT);
     a.out_f32 = 0;
+    sg::set_reciprocals(a);
     const unsigned tiles = (unsigned)(a.n_tiles * a.m_tiles);
 
     if constexpr (SK_ > 1) {   // fp32 partials + self-resetting arrival counters, allocated once
