@@ -142,6 +142,14 @@ def main():
                   % (name, n, k, grid, period_ev, med["period"], med["gap"], med["span"], med["spread"], med["issue"], med["land_med"],
                      med["land_max"], med["stream"], med["epi"], med["wg_med"], med["wg_max"], med["tail"], med["mhz"],
                      sg.api.tuning_as_dict(t_choice)), flush=True)
+            # does the finish time depend on the XCD?  per XCC_ID: median and latest workgroup end after the launch's first entry
+            xcc = (t[4:, :, 7] >> np.uint64(32)).astype(np.int64) & 0xF
+            rel_end = end[4:] - ent[4:].min(axis=1, keepdims=True)
+            line = []
+            for x in sorted(set(xcc.ravel().tolist())):
+                sel = rel_end[xcc == x]
+                line.append("xcc%d %.2f/%.2f" % (x, float(np.median(sel)), float(np.median(np.where(xcc == x, rel_end, 0).max(axis=1)))))
+            print("         workgroup end after first entry, median / median-of-latest per XCD: " + "  ".join(line), flush=True)
             del wb, buf
         return
 
