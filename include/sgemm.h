@@ -90,6 +90,9 @@ size_t sg_workspace_bytes(void);
  *            waves, as in the reference.
  *   split_k  K is also split across split_k workgroups; partials meet in the fp32
  *            workspace and the last workgroup to arrive reduces them in split order.
+ *            Honoured with and without producers (with producers a persistent workgroup
+ *            walks (tile, split) work items, as skinny_gemm/skinny_gemm_kernel.cu:44-64
+ *            decodes them); split_k above k / WARPTILE_K is SG_INVALID_CONFIG.
  */
 int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
                    int m, int n, int k, int b_stride, int split_k,

@@ -83,6 +83,21 @@ def lds_ring_fits(m, k, r):
     return r["split_k"] <= max(1, blocks)
 
 
+def pc_ring_fits(m, k, a_producers, b_producers, consumers, b_lanes, qsize, split_k=1):
+    """The producer/consumer ring's resource rules (``sg_skinny_gemm`` with producers > 0): `qsize` slots of
+    b_lanes weight tiles + the activation rows of one 256-byte K block, the consumers' double-buffered
+    reduction scratch, the flag words and 4 KB of slack within LDS; 1..6 weight tiles per block; no more
+    K splits than K blocks."""
+    if k % 256 or not 1 <= b_lanes <= 6 or min(a_producers, b_producers, consumers, qsize) < 1:
+        return False
+    m_blocks = 1 if m <= 16 else 2
+    xu = _activation_instructions(m, m_blocks)
+    slot = (b_lanes * 4 + xu) * 1024
+    flags = -(-((2 * b_lanes * qsize + 2) * 4) // 1024) * 1024
+    lds = qsize * slot + 2 * b_lanes * m_blocks * consumers * 1024 + flags + 4096
+    return lds <= LDS_USABLE and 1 <= split_k <= k // 256
+
+
 def mid_fits(k, r):
     """Mid-batch kernel: `depth` weight slots of 16*row_tiles*(waves/2) rows and `k_chunks` (or depth)
     activation slots of 32*m_blocks rows, 128 bytes of K each."""

@@ -322,6 +322,8 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
 // Producer/consumer ring: a_producers + b_producers + consumers waves per persistent workgroup.
 struct RingConfig {
     int mt, b_lanes, qsize, a_producers, b_producers, consumers, nt;
+    int split_k = 1;                       // work items per output tile, splitting K among themselves
+    const Workspace* fixed_ws = nullptr;   // split-K partials and counters to use instead of the stream's own workspace
 };
 
 static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
@@ -329,15 +331,29 @@ static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
     if (c.a_producers < 1 || c.b_producers < 1 || c.consumers < 1 || c.qsize < 1) return SG_INVALID_CONFIG;
     if (c.a_producers + c.b_producers + c.consumers > 16) return SG_TOO_MANY_WARPS;
     if (c.b_lanes < 1 || c.b_lanes > 6 || (c.mt != 1 && c.mt != 2)) return SG_INVALID_CONFIG;
+    if (c.split_k < 1 || c.split_k > a.k / 256) return SG_INVALID_CONFIG;
     a.waves = c.consumers;
-    a.split_k = 1;
+    a.split_k = c.split_k;
     a.n_tiles = (a.n + 16 * c.b_lanes - 1) / (16 * c.b_lanes);
     a.m_tiles = (a.m + 16 * c.mt - 1) / (16 * c.mt);
     a.ws = nullptr;
     a.counters = nullptr;
     set_reciprocals(a);
-    const size_t tiles = (size_t)a.n_tiles * a.m_tiles;
+    const size_t tiles = (size_t)a.n_tiles * a.m_tiles * c.split_k;   // work items: one K split of one output tile
     if (tiles > 0x7fffffffu) return SG_BAD_ARGUMENT;
+    if (c.split_k > 1) {
+        // fp32 partials [tile][split][fragment][256] and one arrival counter per fragment of every tile
+        const size_t frags = (size_t)c.b_lanes * c.mt, out_tiles = (size_t)a.n_tiles * a.m_tiles;
+        Workspace w;
+        if (c.fixed_ws) {
+            w = *c.fixed_ws;
+            if (out_tiles * frags > w.n_counters || tiles * frags * 1024 > w.partial_bytes) return SG_WORKSPACE_TOO_SMALL;
+        } else if (int rc = get_workspace(stream, tiles * frags * 1024, out_tiles * frags, &w)) {
+            return rc;
+        }
+        a.ws = w.partials;
+        a.counters = w.counters;
+    }
     int xu = 8;
     if (c.mt == 1) {
         const int need = (a.m + 3) / 4;
@@ -820,6 +836,7 @@ int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* sca
         rc.b_producers = B_producers;
         rc.consumers = consumers;
         rc.nt = 1;
+        rc.split_k = split_k;
         StreamArgs ar{};
         ar.A = A; ar.B = B; ar.D = D; ar.scale = scale_tensor;
         ar.m = m; ar.n = n; ar.k = k; ar.b_stride = b_stride;

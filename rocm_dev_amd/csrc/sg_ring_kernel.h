@@ -7,8 +7,12 @@
 //   B producers   fetch one 16-row weight tile ("lane") of a K block into the ring slot
 //   consumers     own whole K blocks: read the activation tile, then every weight tile of the
 //                 block, and issue the MFMAs; each consumer keeps its own fp32 partial tile
-// The grid is persistent: workgroup w walks tiles w, w + grid, ... and the ring, its flags and
-// every role's position simply continue from one tile to the next.
+// The grid is persistent: workgroup w walks work items w, w + grid, ... and the ring, its flags and
+// every role's position simply continue from one item to the next.  A work item is one K split of
+// one output tile (skinny_gemm_kernel.cu:44-64 decodes the same triple from its tile counter): the
+// items of a tile may run on different workgroups, their fp32 partials meet in the split-K
+// workspace, one arrival counter per 16 x 16 fragment, and the wave that arrives last adds them in
+// split order - no barrier that a producer wave would have to join.
 //
 // Ring and flags (layout of skinny_gemm_kernel.cu:27-30).  Block g of the workgroup's running
 // block count lives in slot g % QSIZE.  queue[2*BL*slot] guards the slot's activation tile,
@@ -35,7 +39,7 @@
 namespace sg {
 
 struct RingArgs {
-    StreamArgs g;       // operands and shape; g.waves = consumers, g.split_k = 1
+    StreamArgs g;       // operands and shape; g.waves = consumers; g.counters holds one word per fragment of every tile
     int a_producers;
     int b_producers;
     int consumers;
@@ -90,17 +94,29 @@ __global__ void __launch_bounds__(1024) ring_gemm_kernel(const RingArgs ra) {
     for (int i = threadIdx.x; i < 2 * BL * Q + 2; i += blockDim.x) queue[i] = 0;  // flags + two arrival counters
     __syncthreads();
 
-    const int total_tiles = a.n_tiles * a.m_tiles;
-    const int my_tiles = ((int)blockIdx.x < total_tiles) ? (total_tiles - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    const int total_items = a.n_tiles * a.m_tiles * a.split_k;
+    const int my_items = ((int)blockIdx.x < total_items) ? (total_items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
     const int blocks = a.k >> 8;                 // K blocks per tile
-    const int total_blocks = blocks * my_tiles;  // running block count of this workgroup
     const unsigned ring_lds = lds_addr(ring);
 
-    auto tile_origin = [&](int j, int& m0, int& n0) __attribute__((always_inline)) {
-        const int t = (int)blockIdx.x + j * (int)gridDim.x;
-        n0 = (t % a.n_tiles) * (16 * BL);
-        m0 = (t / a.n_tiles) * (16 * MT);
+    // The j-th work item of this workgroup: its tile, K split and K range.  Items are numbered with the n tiles
+    // fastest, then the splits of a tile, then the m tiles; the last split takes the remainder of K, so items differ
+    // in length and every role walks them with a cursor over the workgroup's running block count.
+    struct Item { int n0, m0, tile_id, split, kb0, cnt; };
+    auto item_at = [&](int j) __attribute__((always_inline)) {
+        Item it;
+        int tile_n, tile_m, b_begin, b_end;
+        decode_tile(a, (int)blockIdx.x + j * (int)gridDim.x, tile_n, it.split, tile_m);
+        split_range(a, blocks, it.split, b_begin, b_end);
+        it.n0 = tile_n * (16 * BL);
+        it.m0 = tile_m * (16 * MT);
+        it.tile_id = tile_m * a.n_tiles + tile_n;
+        it.kb0 = b_begin;
+        it.cnt = b_end - b_begin;
+        return it;
     };
+    int total_blocks = 0;                        // running block count of this workgroup over all its items
+    for (int j = 0; j < my_items; j++) total_blocks += item_at(j).cnt;
 
     const int q4 = lane >> 2, p4 = lane & 3;
     const int src_row = q4 & 3;
@@ -120,13 +136,18 @@ __global__ void __launch_bounds__(1024) ring_gemm_kernel(const RingArgs ra) {
             return is_a ? &queue[2 * BL * slot] : &queue[2 * (BL * slot + (item - gb * BL)) + 1];
         };
         auto phase_of = [&](int item) __attribute__((always_inline)) { return 2 * ((is_a ? item : item / BL) / Q); };
+        // cursor of the issue side: the work item that holds running block gb (gb only ever grows)
+        int cur_j = 0, cur_base = 0;
+        Item cur = my_items > 0 ? item_at(0) : Item{0, 0, 0, 0, 0, 1};
         auto issue = [&](int item) __attribute__((always_inline)) {
             const int gb = is_a ? item : item / BL;
             const int ln = is_a ? 0 : item - gb * BL;
-            const int j = gb / blocks;
-            const int kb = gb - j * blocks;
-            int m0, n0;
-            tile_origin(j, m0, n0);
+            while (gb >= cur_base + cur.cnt) {
+                cur_base += cur.cnt;
+                cur = item_at(++cur_j);
+            }
+            const int kb = cur.kb0 + (gb - cur_base);
+            const int m0 = cur.m0, n0 = cur.n0;
             const unsigned slot = ring_lds + (unsigned)(gb % Q) * SLOT_BYTES;
             const size_t koff = ((size_t)kb << 8) + src_col;
             if (is_a) {
@@ -179,9 +200,44 @@ __global__ void __launch_bounds__(1024) ring_gemm_kernel(const RingArgs ra) {
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) acc[ln][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    for (int j = 0; j < my_tiles; j++) {
-        // blocks of tile j: running indices j*blocks .. (j+1)*blocks - 1; mine are those = c (mod C)
-        const int gb_lo = j * blocks, gb_hi = gb_lo + blocks;
+    // One finished fragment of work item `it` (already summed over this workgroup's consumers).  Unsplit: scale,
+    // round, store.  Split: the partial goes to the workspace with agent-scope stores (past this XCD's L2), the wave
+    // waits for their acknowledgement and then bumps the fragment's arrival counter; the wave that finds split_k - 1
+    // earlier arrivals reads all partials back in split order, stores the result and zeroes the counter again.
+    auto finish = [&](const Item& it, int f, f32x4 v) __attribute__((always_inline)) {
+        const int m_idx = it.m0 + (f % MT) * 16 + r, n_idx = it.n0 + (f / MT) * 16 + 4 * g16;
+        if (a.split_k == 1) {
+            store_fragment(a, v, scale, m_idx, n_idx);
+            return;
+        }
+        float* tile_ws = a.ws + ((size_t)it.tile_id * a.split_k) * (FRAGS * 256);
+        float* p = tile_ws + ((size_t)it.split * FRAGS + f) * 256 + lane;
+#pragma unroll
+        for (int e = 0; e < 4; e++) __hip_atomic_store(p + e * 64, v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        unsigned* counter = a.counters + (size_t)it.tile_id * FRAGS + f;
+        unsigned arrived = 0;
+        if (lane == 0) arrived = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        arrived = __builtin_amdgcn_readfirstlane(arrived);
+        if (arrived != (unsigned)(a.split_k - 1)) return;
+        const float* q = tile_ws + (size_t)f * 256 + lane;
+        f32x4 sum;
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum[e] = __hip_atomic_load(q + e * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int sp = 1; sp < a.split_k; sp++) {
+            const float* qs = q + (size_t)sp * FRAGS * 256;
+#pragma unroll
+            for (int e = 0; e < 4; e++) sum[e] += __hip_atomic_load(qs + e * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        store_fragment(a, sum, scale, m_idx, n_idx);
+        if (lane == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch
+    };
+
+    int gb_lo = 0;   // running block index at which item j starts
+    for (int j = 0; j < my_items; j++) {
+        const Item it = item_at(j);
+        // blocks of item j: running indices gb_lo .. gb_lo + cnt - 1; mine are those = c (mod C)
+        const int gb_hi = gb_lo + it.cnt;
         int gb = gb_lo + ((c - gb_lo % C) + C) % C;
         for (; gb < gb_hi; gb += C) {
             const int slot = gb % Q;
@@ -189,44 +245,48 @@ __global__ void __launch_bounds__(1024) ring_gemm_kernel(const RingArgs ra) {
             const uint8_t* base = ring + (size_t)slot * SLOT_BYTES + rd_off;
             volatile int* fa = &queue[2 * BL * slot];
             flag_wait(fa, full);
-            i64x2 x[MT][4];
+            // the lane's 16-byte pieces of the block's four 64-byte chunks: chunks 0,1 feed the first
+            // 128-byte MFMA, chunks 2,3 the second (same pieces for both operands, as in mma_block_256)
+            i32x8 x[MT][2];
 #pragma unroll
             for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-                for (int kc = 0; kc < 4; kc++)
-                    x[mt][kc] = *reinterpret_cast<const i64x2*>(base + (BL * 4 + mt * 4) * 1024 + kc * 256);
+                for (int h = 0; h < 2; h++) {
+                    const i32x4 lo = *reinterpret_cast<const i32x4*>(base + (BL * 4 + mt * 4) * 1024 + (2 * h) * 256);
+                    const i32x4 hi = *reinterpret_cast<const i32x4*>(base + (BL * 4 + mt * 4) * 1024 + (2 * h + 1) * 256);
+                    x[mt][h] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             flag_store(fa, full + 1);
 #pragma unroll
             for (int ln = 0; ln < BL; ln++) {
                 volatile int* fb = &queue[2 * (BL * slot + ln) + 1];
                 flag_wait(fb, full);
-                i64x2 w[4];
+                i32x8 w[2];
 #pragma unroll
-                for (int kc = 0; kc < 4; kc++) w[kc] = *reinterpret_cast<const i64x2*>(base + ln * 4096 + kc * 256);
+                for (int h = 0; h < 2; h++) {
+                    const i32x4 lo = *reinterpret_cast<const i32x4*>(base + ln * 4096 + (2 * h) * 256);
+                    const i32x4 hi = *reinterpret_cast<const i32x4*>(base + ln * 4096 + (2 * h + 1) * 256);
+                    w[h] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 flag_store(fb, full + 1);
 #pragma unroll
-                for (int kc = 0; kc < 4; kc++)
+                for (int h = 0; h < 2; h++)
 #pragma unroll
-                    for (int mt = 0; mt < MT; mt++) {
-                        acc[ln][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w[kc].x, x[mt][kc].x, acc[ln][mt], 0, 0, 0);
-                        acc[ln][mt] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w[kc].y, x[mt][kc].y, acc[ln][mt], 0, 0, 0);
-                    }
+                    for (int mt = 0; mt < MT; mt++) acc[ln][mt] = mfma_e4m3_16x16x128(w[h], x[mt][h], acc[ln][mt]);
             }
         }
+        gb_lo = gb_hi;
 
-        // tile j is complete for this consumer: sum the consumers' partials in consumer order
-        int m0, n0;
-        tile_origin(j, m0, n0);
+        // item j is complete for this consumer: sum the consumers' partials in consumer order
         if (C == 1) {
 #pragma unroll
-            for (int f = 0; f < FRAGS; f++)
-                store_fragment(a, acc[f / MT][f % MT], scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g16);
+            for (int f = 0; f < FRAGS; f++) finish(it, f, acc[f / MT][f % MT]);
         } else {
-            // Consumer-only rendezvous (producers are busy with the next tiles and must not be
+            // Consumer-only rendezvous (producers are busy with the next items and must not be
             // stalled by a workgroup barrier): each consumer publishes its partial, then bumps an
-            // arrival counter that only ever counts up; buffer and counter alternate by tile parity.
+            // arrival counter that only ever counts up; buffer and counter alternate by item parity.
             f32x4* buf = red + (size_t)(j & 1) * (FRAGS * C * 64);
 #pragma unroll
             for (int f = 0; f < FRAGS; f++) buf[(f * C + c) * 64 + lane] = acc[f / MT][f % MT];
@@ -237,7 +297,7 @@ __global__ void __launch_bounds__(1024) ring_gemm_kernel(const RingArgs ra) {
             for (int f = c; f < FRAGS; f += C) {
                 f32x4 v = buf[(f * C) * 64 + lane];
                 for (int w = 1; w < C; w++) v += buf[(f * C + w) * 64 + lane];
-                store_fragment(a, v, scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g16);
+                finish(it, f, v);
             }
         }
 #pragma unroll

@@ -9,6 +9,8 @@ import pytest
 import torch
 
 from gpu_util import GEMM_TOL, bits, dev, gemm_tol, scale_tensor
+from launch_rules import expect_lds, expect_mid
+from rocm_dev_amd.autotune import pc_ring_fits, record
 
 pytestmark = pytest.mark.gpu
 
@@ -142,9 +144,10 @@ def test_lds_ring_engine(sg, oracle, cfg, shape):
     rc = sg.skinny_gemm_tuned(A, B, D, S, engine=2, split_k=split_k, waves=waves, row_tiles=row_tiles, depth=depth,
                               non_temporal=nt)
     torch.cuda.synchronize()
-    if rc == 6:
-        pytest.skip("configuration not compiled / does not fit LDS")
-    assert rc == 0, sg.strerror(rc)
+    want = expect_lds(m, n, k, record(2, split_k, waves, row_tiles, 1 if m <= 16 else 2, depth, 4, nt))
+    assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
+    if rc != 0:
+        pytest.skip("the configuration does not fit this shape (LDS, vmcnt or registers), and the library says so")
     got = bits(D)
     assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
@@ -177,38 +180,35 @@ def test_lds_ring_persistent(sg, oracle, cfg, shape):
     A, B, S = dev(a8), dev(b8), scale_tensor(scale)
     D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     kw = dict(engine=2, waves=waves, row_tiles=row_tiles, depth=depth, persistent_wgs_per_cu=per_cu)
+    mb = 1 if m <= 16 else 2
+
+    def rules(**over):
+        return expect_lds(m, n, k, record(2, 1, waves, row_tiles, mb, depth, 4, 1, over.get("per_cu", per_cu), over.get("wt", 0)))
+
     rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
     torch.cuda.synchronize()
-    if rc == 6:
-        pytest.skip("configuration not compiled / does not fit LDS")
-    assert rc == 0, sg.strerror(rc)
+    assert rc == rules(), "library says %s, the resource rules say %d" % (sg.strerror(rc), rules())
+    if rc != 0:
+        pytest.skip("the configuration does not fit this shape (LDS, vmcnt or registers), and the library says so")
     got = bits(D)
     assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     # the non-persistent kernel sums the same partials in the same order: identical bits
     D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     kw["persistent_wgs_per_cu"] = 0
-    assert sg.skinny_gemm_tuned(A, B, D2, S, **kw) == 0
+    rc = sg.skinny_gemm_tuned(A, B, D2, S, **kw)
     torch.cuda.synchronize()
-    assert np.array_equal(bits(D2), got)
-    # ... and so does the variant that keeps the activations resident in LDS (one activation tile only)
-    if m <= (16 if m <= 16 else 32):
-        D3 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
-        kw.update(persistent_wgs_per_cu=per_cu, wave_tiles=2)
-        rc = sg.skinny_gemm_tuned(A, B, D3, S, **kw)
-        torch.cuda.synchronize()
-        if rc != 6:
-            assert rc == 0, sg.strerror(rc)
-            assert np.array_equal(bits(D3), got)
-    # ... and the variants with a dedicated epilogue wave (same partials, same order)
-    for wave_tiles in (4, 6):
-        if wave_tiles == 6 and m > (16 if m <= 16 else 32):
-            continue
+    assert rc == rules(per_cu=0)
+    if rc == 0:
+        assert np.array_equal(bits(D2), got)
+    # ... and so do the variant that keeps the activations resident in LDS (one activation tile only) and the
+    # variants with a dedicated epilogue wave (same partials, same order)
+    for wave_tiles in (2, 4, 6):
         D4 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
         kw.update(persistent_wgs_per_cu=per_cu, wave_tiles=wave_tiles)
         rc = sg.skinny_gemm_tuned(A, B, D4, S, **kw)
         torch.cuda.synchronize()
-        if rc not in (4, 6):
-            assert rc == 0, sg.strerror(rc)
+        assert rc == rules(wt=wave_tiles), (wave_tiles, sg.strerror(rc), rules(wt=wave_tiles))
+        if rc == 0:
             assert np.array_equal(bits(D4), got)
 
 
@@ -239,12 +239,10 @@ def test_lds_ring_activations_in_registers(sg, oracle, cfg, shape):
     kw = dict(engine=2, waves=waves, row_tiles=row_tiles, depth=depth, persistent_wgs_per_cu=1, wave_tiles=3 + (4 if epi else 0))
     rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
     torch.cuda.synchronize()
-    blocks = k // 256
-    fits = blocks % waves == 0 and (blocks // waves) in (1, 2, 4) and (blocks // waves) * (1 if m <= 16 else 2) <= 4
-    if rc == 6:
-        assert not fits or depth * row_tiles * waves * 4 > 140 or waves + epi > 8, "a configuration that fits was rejected"
-        pytest.skip("configuration does not apply to this shape")
-    assert rc == 0, sg.strerror(rc)
+    want = expect_lds(m, n, k, record(2, 1, waves, row_tiles, 1 if m <= 16 else 2, depth, 4, 1, 1, 3 + (4 if epi else 0)))
+    assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
+    if rc != 0:
+        pytest.skip("configuration does not apply to this shape, and the library says so")
     got = bits(D)
     assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     # same partial sums in the same order as the persistent kernel with the activations in the stage
@@ -284,14 +282,50 @@ def test_producer_consumer_ring(sg, oracle, cfg, shape):
     D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     rc = sg.skinny_gemm(A, B, D, S, 1, ap, bp, cons, bl, qs, op_m, ops)
     torch.cuda.synchronize()
+    fits = pc_ring_fits(m, k, ap, bp, cons, bl, qs)
     if rc == 6:
+        assert not fits, "a ring that fits LDS was rejected"
         pytest.skip("ring does not fit LDS")
+    assert fits, "a ring that does not fit LDS was launched"
     assert rc == 0, sg.strerror(rc)
     got = bits(D)
     assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     for _ in range(3):   # repeated runs are the reference's race probe (bench.py -t N)
         D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
         assert sg.skinny_gemm(A, B, D2, S, 1, ap, bp, cons, bl, qs, op_m, ops) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(D2), got)
+
+
+@pytest.mark.parametrize("split_k", [2, 3, 5])
+@pytest.mark.parametrize("cfg", [(1, 1, 1, 1, 2), (1, 4, 3, 2, 6), (2, 6, 2, 3, 4), (1, 8, 4, 4, 5)])
+@pytest.mark.parametrize("shape", [(8, 64, 256), (8, 512, 4096), (5, 1000, 2048), (32, 4096, 1280), (16, 96, 14336),
+                                   (40, 2048, 768)])
+def test_producer_consumer_ring_split_k(sg, oracle, cfg, shape, split_k):
+    """The ring honours split_k: a persistent workgroup walks (tile, split) work items, the last split takes the
+    remainder of K (skinny_gemm_kernel.cu:44-64), fp32 partials meet in the workspace.  grid.py:158 searches
+    split_k in {2, 3, 5}.  More splits than 256-byte K blocks is refused, not ignored."""
+    ap, bp, cons, bl, qs = cfg
+    m, n, k = shape
+    op_m = 8 if m <= 8 else (16 if m <= 16 else 32)
+    ops = 256 // (512 // op_m)
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=19)
+    ref = oracle.gemm_omp(a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = sg.skinny_gemm(A, B, D, S, split_k, ap, bp, cons, bl, qs, op_m, ops)
+    torch.cuda.synchronize()
+    fits = pc_ring_fits(m, k, ap, bp, cons, bl, qs, split_k)
+    if not fits:
+        assert rc == 6, "split_k=%d on %d K blocks must be refused, got %s" % (split_k, k // 256, sg.strerror(rc))
+        assert np.isnan(oracle.bf16_to_f32(bits(D))).all(), "a refused launch wrote D"
+        return
+    assert rc == 0, sg.strerror(rc)
+    got = bits(D)
+    assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
+    for _ in range(3):   # arrival counters reset themselves: every repeat gives the same bits
+        D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        assert sg.skinny_gemm(A, B, D2, S, split_k, ap, bp, cons, bl, qs, op_m, ops) == 0
         torch.cuda.synchronize()
         assert np.array_equal(bits(D2), got)
 
@@ -397,9 +431,10 @@ def test_mid_batch_engine(sg, oracle, cfg, shape):
     kw = dict(engine=4, split_k=split_k, waves=waves, row_tiles=rgw, m_blocks=mh, depth=depth, k_chunks=dx)
     rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
     torch.cuda.synchronize()
-    if rc == 6:
-        pytest.skip("configuration not compiled / does not fit")
-    assert rc == 0, sg.strerror(rc)
+    want = expect_mid(m, n, k, record(4, split_k, waves, rgw, mh, depth, dx))
+    assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
+    if rc != 0:
+        pytest.skip("no such tile / ring combination, and the library says so")
     got = bits(D)
     assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
@@ -466,9 +501,10 @@ def test_lds_ring_wave_tiles(sg, oracle, cfg, shape):
     kw = dict(engine=2, waves=waves, row_tiles=row_tiles, depth=depth, persistent_wgs_per_cu=per_cu, wave_tiles=1)
     rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
     torch.cuda.synchronize()
-    if rc == 6:
-        pytest.skip("configuration not compiled / does not fit LDS")
-    assert rc == 0, sg.strerror(rc)
+    want = expect_lds(m, n, k, record(2, 1, waves, row_tiles, 1 if m <= 16 else 2, depth, 4, 1, per_cu, 1))
+    assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
+    if rc != 0:
+        pytest.skip("the configuration does not fit this shape (LDS, vmcnt or registers), and the library says so")
     got = bits(D)
     assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")

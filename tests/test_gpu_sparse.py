@@ -9,6 +9,8 @@ import pytest
 import torch
 
 from gpu_util import GEMM_TOL, bits, dev, gemm_tol, scale_tensor
+from launch_rules import expect_sparse
+from rocm_dev_amd.autotune import record
 
 pytestmark = pytest.mark.gpu
 
@@ -80,9 +82,10 @@ def test_sparse_tuned_configs(sg, oracle, cfg, shape):
     ref = oracle.gemm_sparse24(a8, vals, meta, scale)
     t = sg.SgTuning(2, split_k, waves, row_tiles, 1 if m <= 16 else 2, depth, 8, 1, 0)
     rc, got = _run(sg, a8, vals, meta, scale, tuning=t)
-    if rc == 6:
-        pytest.skip("configuration not compiled / does not fit LDS")
-    assert rc == 0, sg.strerror(rc)
+    want = expect_sparse(m, n, k, record(2, split_k, waves, row_tiles, 1 if m <= 16 else 2, depth))
+    assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
+    if rc != 0:
+        pytest.skip("the configuration does not fit this shape, and the library says so")
     assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     rc, again = _run(sg, a8, vals, meta, scale, tuning=t)
     assert rc == 0 and np.array_equal(again, got)
@@ -111,9 +114,10 @@ def test_sparse_wave_per_tile_configs(sg, oracle, cfg, shape):
     ref = oracle.gemm_sparse24(a8, vals, meta, scale)
     t = sg.SgTuning(2, 1, waves, row_tiles, 1, depth, 8, 1, per_cu, 1)
     rc, got = _run(sg, a8, vals, meta, scale, tuning=t)
-    if rc == 6:
-        pytest.skip("configuration not compiled / does not fit LDS")
-    assert rc == 0, sg.strerror(rc)
+    want = expect_sparse(m, n, k, record(2, 1, waves, row_tiles, 1, depth, 8, 1, per_cu, 1))
+    assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
+    if rc != 0:
+        pytest.skip("the configuration does not fit this shape, and the library says so")
     assert oracle.max_rel_err_bf16(got, ref) <= gemm_tol(k)
     rc, again = _run(sg, a8, vals, meta, scale, tuning=t)
     assert rc == 0 and np.array_equal(again, got)
