@@ -44,19 +44,20 @@ def test_fixtures_gpu(oracle):
     import torch
 
     import rocm_dev_amd as sg
-    from gpu_util import bits, dev, gemm_tol, scale_tensor
+    from gpu_util import GEMM_TOL, bits, dev, gemm_reference, scale_tensor, sparse_reference
 
     z = np.load(os.path.join(GOLD, "gemm_8x64x512.npz"))
     D = torch.empty((8, 64), dtype=torch.bfloat16, device="cuda")
     assert sg.skinny_gemm_fastpath(dev(z["a8"]), dev(z["b8"]), D, scale_tensor(z["scale"])) == 0
     torch.cuda.synchronize()
-    assert oracle.max_rel_err_bf16(bits(D), z["d_bf16"]) <= gemm_tol(512)
+    # k = 512: against the oracle's model of the instruction's summation (gpu_util.gemm_reference says why)
+    assert oracle.max_rel_err_bf16(bits(D), gemm_reference(oracle, z["a8"], z["b8"], z["scale"])) <= GEMM_TOL
 
     s = np.load(os.path.join(GOLD, "sparse24_8x32x512.npz"))
     D = torch.empty((8, 32), dtype=torch.bfloat16, device="cuda")
     assert sg.sparse24_gemm(dev(s["a8"]), dev(s["vals"]), dev(s["meta"]), D, scale_tensor(s["scale"])) == 0
     torch.cuda.synchronize()
-    assert oracle.max_rel_err_bf16(bits(D), s["d_bf16"]) <= gemm_tol(512)
+    assert oracle.max_rel_err_bf16(bits(D), sparse_reference(oracle, s["a8"], s["vals"], s["meta"], s["scale"])) <= GEMM_TOL
 
     c = np.load(os.path.join(GOLD, "codec_2x16x256.npz"))
     Q = torch.empty((2, 16, 256), dtype=torch.uint8, device="cuda")

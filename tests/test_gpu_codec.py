@@ -75,6 +75,32 @@ def test_encode_decode_reduce_config3_slice(sg, oracle):
     assert oracle.max_rel_err_bf16(got, oracle.bf16_from_f32(truth.astype(np.float32))) <= GEMM_TOL
 
 
+def test_encode_reduce_config3_full_size(sg, oracle):
+    """benchmark configuration 3 at full size, the seeded recipe itself: eight 8192 x 8192 bf16 buffers from the
+    oracle's generator (N(0,1), 0.1 % of the entries +-50), encoded per row, then decoded and summed in fp32.
+    Codes, scales and the reduced bf16 output must equal the oracle's bit for bit."""
+    nbuf, rows, cols = 8, 8192, 8192
+    Q = torch.empty((nbuf, rows, cols), dtype=torch.uint8, device="cuda")
+    S = torch.empty((nbuf, rows), dtype=torch.float32, device="cuda")
+    q_ref = np.empty((nbuf, rows, cols), np.uint8)
+    s_ref = np.empty((nbuf, rows), np.float32)
+    for i in range(nbuf):
+        X = oracle.normal_bf16_outliers((rows, cols), seed=i, stream_id=3, frac=0.001, mag=50.0)
+        assert sg.fp8_encode_rows(dev(X), Q[i], S[i]) == 0
+        q_ref[i], s_ref[i] = oracle.fp8_encode_rows(X)
+        torch.cuda.synchronize()
+        assert np.array_equal(S[i].cpu().numpy(), s_ref[i]), i
+        assert np.array_equal(Q[i].cpu().numpy(), q_ref[i]), i
+    del X
+    Y = torch.empty((rows, cols), dtype=torch.bfloat16, device="cuda")
+    assert sg.fp8_reduce_rows(Q, S, Y) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(Y), oracle.fp8_reduce_rows(q_ref, s_ref))
+    assert sg.fp8_decode_rows(Q[7], S[7], Y) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(Y), oracle.fp8_decode_rows(q_ref[7], s_ref[7]))
+
+
 @pytest.mark.parametrize("nbuf", [1, 2, 3, 4, 5])
 def test_reduce_other_counts(sg, oracle, nbuf):
     rows, cols = 40, 1040 // 16 * 16

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_util import bits, dev, gemm_tol, scale_tensor
+from gpu_util import GEMM_TOL, bits, dev, gemm_reference, scale_tensor
 from rocm_dev_amd import autotune
 
 pytestmark = pytest.mark.gpu
@@ -48,18 +48,18 @@ def _tuned(sg, A, B, S, m, n, r):
 def test_fastpath_launches_the_stored_record(sg, oracle, shape, rec):
     m, n, k = shape
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=5)
-    ref = oracle.gemm_omp(a8, b8, scale)
+    ref = gemm_reference(oracle, a8, b8, scale)
     A, B, S = dev(a8), dev(b8), scale_tensor(scale)
     before = _fast(sg, A, B, S, m, n)
     explicit = _tuned(sg, A, B, S, m, n, rec)
-    assert oracle.max_rel_err_bf16(explicit, ref) <= gemm_tol(k)
+    assert oracle.max_rel_err_bf16(explicit, ref) <= GEMM_TOL
     sg.tuning_set(m, n, k, _record(sg, rec))
     choice, from_table = sg.skinny_gemm_choice(m, n, k)
     assert from_table and {f: getattr(choice, f) for f in autotune.FIELDS} == rec
     after = _fast(sg, A, B, S, m, n)
     # every reduction in the library has a fixed order, so the same record gives the same bits
     assert np.array_equal(after, explicit)
-    assert oracle.max_rel_err_bf16(after, ref) <= gemm_tol(k)
+    assert oracle.max_rel_err_bf16(after, ref) <= GEMM_TOL
     # the row/column-scaled entry point goes through the same choice
     D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     assert sg.skinny_gemm_rowcol(A, B, D, S) == 0
@@ -88,7 +88,7 @@ def test_unusable_record_falls_back(sg, oracle, rec):
     after = _fast(sg, A, B, S, m, n)
     if rc != 0:
         assert np.array_equal(after, before)
-    assert oracle.max_rel_err_bf16(after, oracle.gemm_omp(a8, b8, scale)) <= gemm_tol(k)
+    assert oracle.max_rel_err_bf16(after, gemm_reference(oracle, a8, b8, scale)) <= GEMM_TOL
 
 
 def test_driver_measures_checks_and_writes_a_loadable_table(sg, oracle, tmp_path, capsys):
@@ -97,11 +97,11 @@ def test_driver_measures_checks_and_writes_a_loadable_table(sg, oracle, tmp_path
     assert ran > 10 and 1 <= len(kept) <= 3 and base_us > 0
     assert [us for us, _ in kept] == sorted(us for us, _ in kept)
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=7)
-    ref = oracle.gemm_omp(a8, b8, scale)
+    ref = gemm_reference(oracle, a8, b8, scale)
     A, B, S = dev(a8), dev(b8), scale_tensor(scale)
     for us, rec in kept:
         assert rec in autotune.search_space(m, n, k) and 0 < us < 1e4
-        assert oracle.max_rel_err_bf16(_tuned(sg, A, B, S, m, n, rec), ref) <= gemm_tol(k)
+        assert oracle.max_rel_err_bf16(_tuned(sg, A, B, S, m, n, rec), ref) <= GEMM_TOL
     out = tmp_path / "tuning.txt"
     assert autotune.main(["--shapes", "%dx%dx%d" % (m, n, k), "64x512x1024", "--out", str(out), "--launches", "8",
                           "--limit", "24", "--min-gain", "-1"]) == 0          # -1: always keep the winner
@@ -109,4 +109,4 @@ def test_driver_measures_checks_and_writes_a_loadable_table(sg, oracle, tmp_path
     assert set(entries) == {(m, n, k), (64, 512, 1024)} and entries[(64, 512, 1024)]["engine"] == 4
     sg.tuning_load(out)
     assert sg.tuning_count() == 2
-    assert oracle.max_rel_err_bf16(_fast(sg, A, B, S, m, n), ref) <= gemm_tol(k)
+    assert oracle.max_rel_err_bf16(_fast(sg, A, B, S, m, n), ref) <= GEMM_TOL
