@@ -33,4 +33,5 @@ from .api import (  # noqa: F401
     tuning_save,
     tuning_set,
 )
+from . import synth  # noqa: F401
 from .build import build  # noqa: F401
