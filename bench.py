@@ -474,6 +474,37 @@ def main():
         others["tiled_sum_reduce_8x1024x8192"] = {"us": round(tsr_us, 2), "TBps": round(tsr_bytes / tsr_us / 1e6, 3),
                                                   "note": "reads 512 MiB per launch (beyond the 256 MB cache), writes 32 MiB"}
         del ta, tbb, td
+        # bf16 activations quantised per row inside the GEMM (one launch) against the two launches it replaces
+        # (sg_fp8_encode_rows, then sg_skinny_gemm_rowcol with the library's own configuration), cold weights
+        fused_rows = []
+        for name in order:
+            n, k = SHAPES[name]
+            for m in (8, 16):
+                xb = synth.normal_f32((m, k), 1, 1).bfloat16()
+                q = torch.empty((m, k), device="cuda", dtype=torch.uint8)
+                rs = torch.empty((m,), device="cuda", dtype=torch.float32)
+                cs = torch.ones((n,), device="cuda", dtype=torch.float32)
+                d = outs[(name, m)]
+                w = weights[name]
+                _, is_fused = sg.skinny_gemm_bf16act_choice(m, n, k)
+
+                def one(i, st):
+                    rc = lib.sg_skinny_gemm_bf16act(xb.data_ptr(), w[i % len(w)].data_ptr(), d.data_ptr(), scl[(name, m)].data_ptr(),
+                                                    cs.data_ptr(), None, m, n, k, k, st)
+                    if rc != 0:
+                        raise RuntimeError("sg_skinny_gemm_bf16act: %s" % sg.strerror(rc))
+
+                def two(i, st):
+                    rc = lib.sg_fp8_encode_rows(xb.data_ptr(), q.data_ptr(), rs.data_ptr(), m, k, st)
+                    rc = rc or lib.sg_skinny_gemm_rowcol(q.data_ptr(), w[i % len(w)].data_ptr(), d.data_ptr(), scl[(name, m)].data_ptr(),
+                                                         rs.data_ptr(), cs.data_ptr(), m, n, k, k, st)
+                    if rc != 0:
+                        raise RuntimeError("encode_rows + rowcol: %s" % sg.strerror(rc))
+
+                fused_rows.append({"shape": name, "m": m, "n": n, "k": k, "single_launch": bool(is_fused),
+                                   "bf16act_us": round(graph_time_us(one, 40), 3),
+                                   "encode_then_rowcol_us": round(graph_time_us(two, 40), 3)})
+        others["bf16_activations"] = fused_rows
         # 2:4 sparse GEMMs
         sp = []
         for (n, k) in ((4096, 14336), (14336, 4096)):

@@ -160,6 +160,32 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const
 int sg_skinny_gemm_tuned_noalloc(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
                                  int m, int n, int k, int b_stride, const SgTuning* tuning, void* stream);
 
+/* The rowcol GEMM on bf16 activations: the per-row quantisation of sg_fp8_encode_rows happens inside the GEMM,
+ * so a decode layer's "quantise activations, then project" is one launch instead of two.
+ *     s[i]    = absmax(X[i,:]) / 448  (1 for an all-zero row);   A[i][k] = e4m3_rne_sat(fp32(X[i][k]) / s[i])
+ *     D[i][j] = bf16( ((sum_k A[i][k]*B[j][k]) * scale) * s[i] * col_scales[j] )
+ * - bit for bit what sg_fp8_encode_rows followed by sg_skinny_gemm_rowcol(row_scales = its scales) returns when
+ * both run the same GEMM configuration.  No counterpart in the reference, whose A producer copies FP8 bytes
+ * (skinny_gemm/producers/producers.cuh:5-25) and whose epilogue applies one scalar
+ * (skinny_gemm/consumers/mfma_16x16x32_consumer.cu:111-118).  X is [m][k] bf16, 16-byte aligned; scale_tensor
+ * and col_scales may be NULL (factor 1); row_scales_out, if not NULL, receives s[0..m).
+ * The fused kernel applies where one activation tile covers m (m <= 32), k % 256 == 0 and the codes fit LDS beside
+ * the weight rings of four waves: every workgroup quantises its own copy of the activations while its first weight
+ * stages are in flight.  That repeats the quantisation in every workgroup, so the library uses it only where it
+ * measured faster than the two launches - m <= 8 and at least three 16-row tiles per CU (8 x 28672 x 4096: 26.9
+ * against 29.0 us) - and otherwise runs the two launches itself, with the codes in a per-stream scratch buffer it
+ * keeps.  sg_skinny_gemm_bf16act_choice says which (*fused) and with which record.  sg_skinny_gemm_bf16act_tuned
+ * always runs the fused kernel: with the given record (LDS ring, persistent_wgs_per_cu >= 1, wave_tiles 2 or 6,
+ * row_tiles 1, depth 2; at most 8 streaming waves), or - engine 0 - the library's own for the shape;
+ * SG_INVALID_CONFIG where the kernel does not apply. */
+int sg_skinny_gemm_bf16act(const void* X_bf16, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                           const float* col_scales, float* row_scales_out, int m, int n, int k, int b_stride,
+                           void* stream);
+int sg_skinny_gemm_bf16act_tuned(const void* X_bf16, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                                 const float* col_scales, float* row_scales_out, int m, int n, int k, int b_stride,
+                                 const SgTuning* tuning, void* stream);
+int sg_skinny_gemm_bf16act_choice(int m, int n, int k, SgTuning* out, int* fused);
+
 /* The configuration sg_skinny_gemm_auto would use, for logging and tuning drivers.
  * out[8] = {split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops}. */
 int sg_skinny_gemm_pick(int m, int n, int k, int out[8]);

@@ -20,6 +20,8 @@ from .api import (  # noqa: F401
     skinny_gemm_choice,
     skinny_gemm_pick,
     skinny_gemm_rowcol,
+    skinny_gemm_bf16act,
+    skinny_gemm_bf16act_choice,
     skinny_gemm_tuned,
     skinny_gemm_tuned_noalloc,
     init_stream,

@@ -26,6 +26,9 @@ SIGNATURES = {
     "sg_skinny_gemm_fastpath": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "sg_skinny_gemm_auto": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm_rowcol": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "sg_skinny_gemm_bf16act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "sg_skinny_gemm_bf16act_tuned": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
+    "sg_skinny_gemm_bf16act_choice": (_i, [_i, _i, _i, _vp, C.POINTER(_i)]),
     "sg_skinny_gemm_tuned": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sg_skinny_gemm_tuned_noalloc": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "sg_skinny_gemm_pick": (_i, [_i, _i, _i, C.POINTER(_i * 8)]),

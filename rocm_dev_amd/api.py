@@ -121,6 +121,38 @@ def skinny_gemm_rowcol(A, B, D, scale_tensor=None, row_scales=None, col_scales=N
     return _done(rc, check)
 
 
+def skinny_gemm_bf16act(X, B, D, scale_tensor=None, col_scales=None, row_scales_out=None, tuning=None, check=False):
+    """The rowcol GEMM on bf16 activations X [m, k]: rows quantised to E4M3 inside the GEMM (as fp8_encode_rows would),
+    D = bf16(((q(X) @ B^T) * scale) * row_scale[:, None] * col_scales[None, :]); row_scales_out, if given, receives the
+    row scales.  One launch where the fused kernel pays (skinny_gemm_bf16act_choice), two inside the library otherwise;
+    with `tuning` (an SgTuning; engine 0 = the library's record for the shape) always the fused kernel."""
+    m, k = X.shape
+    n = B.shape[0]
+    if col_scales is not None and tuple(col_scales.shape) != (n,):
+        raise ValueError("col_scales must have shape (n,)")
+    if row_scales_out is not None and tuple(row_scales_out.shape) != (m,):
+        raise ValueError("row_scales_out must have shape (m,)")
+    args = (_dev(X, torch.bfloat16), _dev(B, *_FP8), _dev(D, torch.bfloat16),
+            None if scale_tensor is None else _dev(scale_tensor, torch.float32),
+            None if col_scales is None else _dev(col_scales, torch.float32),
+            None if row_scales_out is None else _dev(row_scales_out, torch.float32), m, n, k, B.stride(0))
+    with torch.cuda.device(X.device):
+        if tuning is None:
+            rc = lib.sg_skinny_gemm_bf16act(*args, _stream())
+        else:
+            rc = lib.sg_skinny_gemm_bf16act_tuned(*args, C.byref(tuning), _stream())
+    return _done(rc, check)
+
+
+def skinny_gemm_bf16act_choice(m, n, k):
+    """(record, fused): the SgTuning skinny_gemm_bf16act launches for the shape and whether it is the fused kernel."""
+    t, fused = SgTuning(), C.c_int(0)
+    rc = lib.sg_skinny_gemm_bf16act_choice(m, n, k, C.byref(t), C.byref(fused))
+    if rc != 0:
+        raise SgError(rc)
+    return t, bool(fused.value)
+
+
 def skinny_gemm_tuned(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k=1, waves=4, row_tiles=1, m_blocks=None,
                       depth=2, k_chunks=4, non_temporal=1, persistent_wgs_per_cu=0, wave_tiles=0, check=False):
     """The library-native tuning entry (no reference counterpart): pick the engine and its shape."""

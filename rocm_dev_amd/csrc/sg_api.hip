@@ -266,6 +266,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     size_t lds = (size_t)c.waves * c.depth * stage + 4096;
     unsigned grid = (unsigned)(tiles * c.split_k);
     int mode = 0, extra_wave = 0;
+    if (a.A16 && !(c.persist > 0 && (c.wavetile & 3) == 2)) return SG_INVALID_CONFIG;
     if (c.wavetile == 1) {
         // whole activation matrix resident: one tile row of activations only, no K split
         if (c.split_k != 1 || a.m_tiles != 1 || c.persist < 1) return SG_INVALID_CONFIG;
@@ -308,9 +309,13 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         if (want < grid) grid = (unsigned)want;
     }
     if (lds > 159 * 1024) return SG_INVALID_CONFIG;  // 160 KB per CU, minus the kernel's static LDS
+    if (a.A16) {   // only the resident-activation kernel quantises bf16 activations itself
+        if (mode != 3) return SG_INVALID_CONFIG;
+        mode = 4;
+    }
     const unsigned threads = (unsigned)(c.waves + extra_wave) * 64;
     if (threads > 1024) return SG_TOO_MANY_WARPS;
-    if (mode == 0 || mode == 1 || mode == 3) a.stamps = take_stamps(grid);
+    if (mode == 0 || mode == 1 || mode == 3 || mode == 4) a.stamps = take_stamps(grid);
 #define SG_GO(MT, RG)                                                                                          \
     if (c.mt == MT && c.rg == RG)                                                                              \
         return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, mode, a, grid, threads, lds, stream);
@@ -687,6 +692,70 @@ static Config pick_config(int m, int n, int k, int cu_count) {
     return direct_config(m, n, k, cu_count);
 }
 
+// bf16 activations -> the GEMM quantises them itself: the persistent kernel with the activations resident in LDS
+// (every workgroup derives the row scales and the codes of its own copy).  fused_config: what the kernel can run -
+// one activation tile covers all of m and the codes fit LDS next to the rings of at least four waves.
+static bool fused_config(int m, int k, Config* out) {
+    if (k % 256 != 0 || m > 32) return false;
+    Config c;
+    c.engine = ENGINE_LDS;
+    c.mt = m <= 16 ? 1 : 2;
+    c.rg = 1;
+    c.ku = 4;
+    c.depth = 2;
+    c.split_k = 1;
+    c.nt = 1;
+    c.persist = 1;
+    c.wavetile = 2 | 4;          // resident activations + epilogue wave
+    const int blocks = k / 256;
+    const int xu = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
+    const size_t x_res = (size_t)blocks * xu * 1024;
+    // at least four streaming waves: fewer keep too little in flight per CU
+    for (int waves : {8, 6, 4}) {
+        if (x_res + (size_t)waves * (c.depth * 4 + 2 * c.mt) * 1024 + 4096 > 159 * 1024) continue;
+        c.waves = waves;
+        *out = c;
+        return true;
+    }
+    return false;
+}
+
+// ... and where it pays.  Every workgroup repeats the quantisation of all m x k activations (about 2.4 us of vector
+// work per workgroup at m = 8, k = 4096), which is only hidden where the workgroup goes on to stream several tiles:
+// 8 x 28672 x 4096 takes 26.9 us fused against 29.0 us for the two launches, 8 x 4096 x 4096 8.5 against 8.4,
+// 8 x 6144 x 4096 10.8 against 9.9, and at 16 rows or with a share too long for registers the two launches win.
+static bool pick_bf16act(int m, int n, int k, int cu_count, Config* out) {
+    Config c;
+    if (!fused_config(m, k, &c)) return false;
+    const int tiles = (n + 15) / 16, blocks = k / 256;
+    const int xu = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
+    if (m > 8 || tiles < 3 * cu_count || ((blocks + c.waves - 1) / c.waves) * xu > 8) return false;
+    *out = c;
+    return true;
+}
+
+// Scratch for the two-launch form of sg_skinny_gemm_bf16act (shapes the fused kernel does not take): the E4M3 codes
+// and row scales of the activations, one buffer per (device, stream), grown on demand and kept.
+struct ActScratch { uint8_t* p = nullptr; size_t bytes = 0; };
+static std::map<hipStream_t, ActScratch> g_act[kMaxDevices];
+
+static int get_act_scratch(hipStream_t stream, size_t bytes, uint8_t** out) {
+    int dev;
+    if (int rc = current_device(&dev)) return rc;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    ActScratch& sc = g_act[dev][stream];
+    if (sc.bytes < bytes) {
+        const size_t want = round_up_pow2(bytes, 1u << 20);
+        void* p = workspace_alloc(want);    // an outgrown buffer is kept: launches already enqueued may still read it
+        if (!p) return SG_NO_DEVICE;
+        sc.p = static_cast<uint8_t*>(p);
+        sc.bytes = want;
+        g_ws_bytes[dev] += want;
+    }
+    *out = sc.p;
+    return SG_SUCCESS;
+}
+
 static Config config_from_tuning(const SgTuning& t) {
     Config c;
     c.engine = t.engine;
@@ -975,6 +1044,88 @@ int sg_skinny_gemm_rowcol(const uint8_t* A, const uint8_t* B, void* D, const flo
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
     a.out_f32 = 0;
     return launch_chosen(a, dev->cu_count, static_cast<hipStream_t>(stream));
+}
+
+static void config_to_tuning(const Config& c, SgTuning* out) {
+    out->engine = c.engine; out->split_k = c.split_k; out->waves = c.waves; out->row_tiles = c.rg; out->m_blocks = c.mt;
+    out->depth = c.depth; out->k_chunks = c.ku; out->non_temporal = c.nt; out->persistent_wgs_per_cu = c.persist;
+    out->wave_tiles = c.wavetile;
+}
+
+int sg_skinny_gemm_bf16act(const void* X_bf16, const uint8_t* B, void* D, const float* scale_tensor, const float* col_scales,
+                           float* row_scales_out, int m, int n, int k, int b_stride, void* stream) {
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 16 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (int rc = check_pointers(X_bf16, B, D, m, n, k, b_stride)) return rc;
+    if ((reinterpret_cast<uintptr_t>(row_scales_out) | reinterpret_cast<uintptr_t>(col_scales)) & 3u) return SG_BAD_ALIGNMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    StreamArgs a{};
+    a.B = B; a.D = D; a.scale = scale_tensor;   // nullptr = 1.0f
+    a.col_scale = col_scales;
+    a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
+    a.out_f32 = 0;
+    Config c;
+    if (pick_bf16act(m, n, k, dev->cu_count, &c)) {
+        a.A16 = static_cast<const uint16_t*>(X_bf16);
+        a.row_scale_out = row_scales_out;
+        const int rc = launch_config(c, a, st);
+        if (!rejected_before_launch(rc)) return rc;
+        a.A16 = nullptr;
+        a.row_scale_out = nullptr;
+    }
+    // two launches: the row encoder into the stream's scratch, then the GEMM with its scales in the epilogue
+    uint8_t* scratch = nullptr;
+    const size_t q_bytes = ((size_t)m * k + 255) & ~(size_t)255;
+    if (int rc = get_act_scratch(st, q_bytes + (size_t)m * sizeof(float), &scratch)) return rc;
+    float* scales = row_scales_out ? row_scales_out : reinterpret_cast<float*>(scratch + q_bytes);
+    if (int rc = launch_fp8_encode_rows(X_bf16, scratch, scales, m, k, st)) return rc;
+    a.A = scratch;
+    a.row_scale = scales;
+    return launch_chosen(a, dev->cu_count, st);
+}
+
+int sg_skinny_gemm_bf16act_tuned(const void* X_bf16, const uint8_t* B, void* D, const float* scale_tensor,
+                                 const float* col_scales, float* row_scales_out, int m, int n, int k, int b_stride,
+                                 const SgTuning* t, void* stream) {
+    if (!t) return SG_BAD_ARGUMENT;
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 256 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (int rc = check_pointers(X_bf16, B, D, m, n, k, b_stride)) return rc;
+    if ((reinterpret_cast<uintptr_t>(row_scales_out) | reinterpret_cast<uintptr_t>(col_scales)) & 3u) return SG_BAD_ALIGNMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    Config c;
+    if (t->engine == ENGINE_AUTO) {
+        if (!fused_config(m, k, &c)) return SG_INVALID_CONFIG;
+    } else {
+        c = config_from_tuning(*t);
+        if (c.engine != ENGINE_LDS || (c.mt != 1 && c.mt != 2)) return SG_INVALID_CONFIG;
+    }
+    StreamArgs a{};
+    a.A16 = static_cast<const uint16_t*>(X_bf16);
+    a.row_scale_out = row_scales_out;
+    a.B = B; a.D = D; a.scale = scale_tensor;
+    a.col_scale = col_scales;
+    a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
+    a.out_f32 = 0;
+    return launch_config(c, a, static_cast<hipStream_t>(stream));
+}
+
+int sg_skinny_gemm_bf16act_choice(int m, int n, int k, SgTuning* out, int* fused) {
+    if (!out || m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    int cu = 256;
+    if (get_device_info(&dev) == SG_SUCCESS) cu = dev->cu_count;
+    Config c;
+    if (pick_bf16act(m, n, k, cu, &c)) {
+        config_to_tuning(c, out);
+        if (fused) *fused = 1;
+        return SG_SUCCESS;
+    }
+    if (fused) *fused = 0;
+    return sg_skinny_gemm_choice(m, n, k, out, nullptr);
 }
 
 int sg_tuning_set(int m, int n, int k, const SgTuning* t) {

@@ -19,6 +19,7 @@
 // outside that exponent window take the plain IEEE divide.
 #include "sg_device.h"
 #include "sg_host.h"
+#include "sg_quant.h"
 
 namespace sg {
 
@@ -28,14 +29,6 @@ __device__ __forceinline__ uint32_t cvt_bf16x2(float lo, float hi) {
     f32x2 v = {lo, hi};
     bf16x2_t h = __builtin_convertvector(v, bf16x2_t);
     return __builtin_bit_cast(uint32_t, h);
-}
-
-// Both E4M3 NaN codes (0x7f, 0xff) -> 0x7f in all four bytes: the sign of a NaN quotient (NaN input, inf / inf)
-// depends on how the division is carried out, so the encoder's contract fixes it.
-__device__ __forceinline__ uint32_t canonical_nan_codes(int packed) {
-    const uint32_t u = (uint32_t)packed;
-    const uint32_t nan_sign = ((u & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u;   // bit 7 of every byte whose low seven bits are ones
-    return u & ~nan_sign;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -66,12 +59,7 @@ __global__ void __launch_bounds__(256) fp8_encode_rows_kernel(const uint16_t* __
 
     float amax = 0.0f;
 #pragma unroll
-    for (int c = 0; c < CH; c++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            amax = fmaxf(amax, fabsf(bf16_lo(raw[c][j])));
-            amax = fmaxf(amax, fabsf(bf16_hi(raw[c][j])));
-        }
+    for (int c = 0; c < CH; c++) amax = absmax8_bf16(raw[c], amax);
     amax = wave_max(amax);
     const int nw = T >> 6;
     if (nw > 1) {
@@ -81,38 +69,15 @@ __global__ void __launch_bounds__(256) fp8_encode_rows_kernel(const uint16_t* __
         for (int w = 1; w < nw; w++) amax = fmaxf(amax, wmax[w]);
     }
 
-    const float s = (amax == 0.0f) ? 1.0f : __fdiv_rn(amax, 448.0f);
-    if (t == 0) scales[row] = s;
-    const float y = __fdiv_rn(1.0f, s);
-    const uint32_t aexp = (__float_as_uint(amax) >> 23) & 0xffu;
-    const bool fast = (aexp >= 60u && aexp <= 190u);
+    const RowQuant rq = row_quant(amax);
+    if (t == 0) scales[row] = rq.s;
 
     u32x2* qrow = reinterpret_cast<u32x2*>(Q + (size_t)row * cols);
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int idx = c * T + t;
-        float q[8];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const float x0 = bf16_lo(raw[c][j]), x1 = bf16_hi(raw[c][j]);
-            if (fast) {
-                const float q0 = __fmul_rn(x0, y), q1 = __fmul_rn(x1, y);
-                // copysign: for x = -0 the correction step would return +0, the divide gives -0
-                q[2 * j] = copysignf(__fmaf_rn(__fmaf_rn(-s, q0, x0), y, q0), x0);
-                q[2 * j + 1] = copysignf(__fmaf_rn(__fmaf_rn(-s, q1, x1), y, q1), x1);
-            } else {
-                q[2 * j] = __fdiv_rn(x0, s);
-                q[2 * j + 1] = __fdiv_rn(x1, s);
-            }
-        }
-        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
-        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], w0, true);
-        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[4], q[5], 0, false);
-        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(q[6], q[7], w1, true);
-        if (idx < nchunks) {
-            u32x2 out = {canonical_nan_codes(w0), canonical_nan_codes(w1)};
-            __builtin_nontemporal_store(out, qrow + idx);
-        }
+        const u32x2 out = quantize8_bf16(raw[c], rq);
+        if (idx < nchunks) __builtin_nontemporal_store(out, qrow + idx);
     }
 }
 

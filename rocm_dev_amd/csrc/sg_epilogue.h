@@ -19,7 +19,9 @@
 namespace sg {
 
 struct StreamArgs {
-    const uint8_t* A;
+    const uint8_t* A;       // E4M3 activations [m, k] ...
+    const uint16_t* A16;    // ... or bf16 activations that the kernel quantises per row itself (resident-activation kernel only; A unused)
+    float* row_scale_out;   // with A16: optional [m] output of the row scales the kernel derived, or nullptr
     const uint8_t* B;
     void* D;                // bf16 or fp32, [m, n]
     const float* scale;     // device scalar, or nullptr for 1.0f
@@ -96,7 +98,20 @@ __device__ __forceinline__ int blocks_of_wave(const StreamArgs& a, int n_blk, in
 }
 
 // Writes one finished 16(n) x 16(m) fragment: lane owns m = m_base + l%16, n = n_base + 4*(l/16)..+3.
-__device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, float scale, int m_idx, int n_idx) {
+// `lds_row_scale`, when given, is a per-row factor table in LDS (the scales of activations quantised in the kernel)
+// that takes the place of a.row_scale.
+// `col_factors`, when given, holds a.col_scale[n_idx .. n_idx + 3] fetched ahead of time (col_scale_ahead).
+__device__ __forceinline__ f32x4 col_scale_ahead(const StreamArgs& a, int n_idx) {
+    f32x4 c = {1.0f, 1.0f, 1.0f, 1.0f};
+    if (a.col_scale) {
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (n_idx + e < a.n) c[e] = a.col_scale[n_idx + e];
+    }
+    return c;
+}
+__device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, float scale, int m_idx, int n_idx,
+                                               const float* lds_row_scale = nullptr, const f32x4* col_factors = nullptr) {
     // Pin the fragment before the lane-divergent exit below.  An MFMA needs every lane of the wave
     // (it reads all lanes' operand registers), but the compiler is free to sink the loads and the
     // MFMA that produce `v` into the region where only lanes with m_idx < m are active - it did so
@@ -105,11 +120,12 @@ __device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, flo
     if (m_idx >= a.m) return;
     // scale, then the row factor, then the column factors: three separately rounded fp32 products
     v *= scale;
-    if (a.row_scale) v *= a.row_scale[m_idx];
+    if (lds_row_scale) v *= lds_row_scale[m_idx];
+    else if (a.row_scale) v *= a.row_scale[m_idx];
     if (a.col_scale) {
 #pragma unroll
         for (int e = 0; e < 4; e++)
-            if (n_idx + e < a.n) v[e] *= a.col_scale[n_idx + e];
+            if (n_idx + e < a.n) v[e] *= col_factors ? (*col_factors)[e] : a.col_scale[n_idx + e];
     }
     const size_t off = (size_t)m_idx * a.n + n_idx;
     if (a.out_f32) {

@@ -11,10 +11,11 @@ namespace sg {
 
 template <int XU, int DEPTH, bool NT, int MODE>
 static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
-    if (threads > (unsigned)(MODE == 0 ? lds_launch_bound(SG_MT, SG_RG) : lds_persistent_launch_bound(SG_MT, SG_RG)))
-        return SG_INVALID_CONFIG;
+    constexpr int bound = MODE == 4 ? kQuantThreads : (MODE == 0 ? lds_launch_bound(SG_MT, SG_RG) : lds_persistent_launch_bound(SG_MT, SG_RG));
+    if (threads > (unsigned)bound) return SG_INVALID_CONFIG;
     void (*kernel)(const StreamArgs) = nullptr;
-    if constexpr (MODE == 2) kernel = lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
+    if constexpr (MODE == 4) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true, true>;
+    else if constexpr (MODE == 2) kernel = lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
     else if constexpr (MODE == 3) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
     else if constexpr (MODE == 1) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false>;
     else kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
@@ -27,6 +28,13 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
 #define SG_CASE(XU_, DEPTH_)                                                                    \
     if (xu == XU_ && depth == DEPTH_) {                                                         \
         if constexpr (XU_ <= 4 * SG_MT && (SG_MT == 1 || XU_ > 4)) {                            \
+            if (mode == 4) { /* bf16 activations quantised in the kernel: one row tile per wave, two slots */ \
+                if constexpr (SG_RG == 1 && DEPTH_ == 2)                                        \
+                    return nt ? launch_one<XU_, DEPTH_, true, 4>(a, grid, threads, lds, stream) \
+                              : launch_one<XU_, DEPTH_, false, 4>(a, grid, threads, lds, stream); \
+                else                                                                            \
+                    return SG_INVALID_CONFIG;                                                   \
+            }                                                                                   \
             if (mode == 2 || mode == 3) {                                                       \
                 if constexpr ((DEPTH_ - 1) * (SG_RG * 4) <= 63) {                               \
                     if (mode == 3)                                                              \

@@ -31,6 +31,7 @@
 
 #include "sg_device.h"
 #include "sg_epilogue.h"
+#include "sg_quant.h"
 
 namespace sg {
 
@@ -249,6 +250,122 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     stamps.end(a);
 }
 
+// bf16 activations -> E4M3 codes in the resident-activation layout of the persistent kernel, quantised per row
+// exactly as sg_fp8_encode_rows does (same arithmetic, sg_quant.h), by the workgroup that is about to use them.
+// Replaces the activation DMA of the resident kernel: K block kb is handled by wave kb % waves (the only wave that
+// will read it), and lane l of "instruction" u produces the 16 bytes the DMA would have put at (kb*XU + u) KB + 16*l:
+// row 4u + (l/4)%4, k = 256 kb + 64 (l/16) + 16 ((l + u) % 4) .. +15.
+//
+// Order of events: the wave loads its share of the bf16 activations and takes the row maxima of it (load_and_max);
+// the caller then issues the prologue DMAs of the weight ring; finish() combines the maxima of all waves (one
+// barrier), derives the scales and writes the codes - while the weights are arriving.  A wave keeps at most 8 chunks
+// of 16 values in registers between the two steps (64 registers); a larger share - long K - is read a second time
+// (from L2).  Every wave of the workgroup calls both steps exactly once; the caller's next barrier publishes the
+// codes and `xscale`.
+template <int XU>
+struct ActivationQuantizer {
+    static constexpr int KB_MAX = XU >= 8 ? 1 : 8 / XU;   // K blocks of a wave whose chunks fit 64 registers
+    u32x4 raw[KB_MAX][XU][2];
+    float pm[XU];
+    int row[XU];
+    unsigned koff[XU];
+    int kb0, nkb, rr;
+
+    __device__ __forceinline__ const u32x4* chunk(const StreamArgs& a, int kb, int u) const {
+        return reinterpret_cast<const u32x4*>(a.A16 + (size_t)row[u] * a.k + ((size_t)kb << 8) + koff[u]);
+    }
+
+    __device__ __forceinline__ void load_and_max(const StreamArgs& a, int blocks, int waves, int wave, int lane) {
+        rr = (lane >> 2) & 3;
+        const int col = (lane >> 4) * 64;
+#pragma unroll
+        for (int u = 0; u < XU; u++) {
+            const int r = 4 * u + rr;
+            row[u] = r < a.m ? r : a.m - 1;          // rows past the edge repeat the last row, as the DMA does
+            koff[u] = col + (((lane & 3) + (u & 3)) & 3) * 16;
+            pm[u] = 0.0f;
+        }
+        kb0 = wave < waves ? wave : blocks;
+        nkb = kb0 < blocks ? (blocks - kb0 + waves - 1) / waves : 0;
+        if (nkb <= KB_MAX) {
+#pragma unroll
+            for (int i = 0; i < KB_MAX; i++)
+#pragma unroll
+                for (int u = 0; u < XU; u++) {
+                    raw[i][u][0] = raw[i][u][1] = u32x4{0u, 0u, 0u, 0u};
+                    if (i < nkb) {
+                        const u32x4* src = chunk(a, kb0 + i * waves, u);
+                        raw[i][u][0] = src[0];
+                        raw[i][u][1] = src[1];
+                    }
+                }
+#pragma unroll
+            for (int i = 0; i < KB_MAX; i++)
+#pragma unroll
+                for (int u = 0; u < XU; u++) pm[u] = absmax8_bf16(raw[i][u][1], absmax8_bf16(raw[i][u][0], pm[u]));
+        } else {
+            for (int kb = kb0; kb < blocks; kb += waves)
+#pragma unroll
+                for (int u = 0; u < XU; u++) {
+                    const u32x4* src = chunk(a, kb, u);
+                    pm[u] = absmax8_bf16(src[1], absmax8_bf16(src[0], pm[u]));
+                }
+        }
+    }
+
+    __device__ __forceinline__ void finish(const StreamArgs& a, uint8_t* xres, float* wmax, float* xscale, int blocks, int waves,
+                                           int wave, int lane) {
+        // lanes that share a row for a given u differ in lane bits 0, 1, 4, 5
+#pragma unroll
+        for (int u = 0; u < XU; u++) {
+            pm[u] = fmaxf(pm[u], __shfl_xor(pm[u], 1));
+            pm[u] = fmaxf(pm[u], __shfl_xor(pm[u], 2));
+            pm[u] = fmaxf(pm[u], __shfl_xor(pm[u], 16));
+            pm[u] = fmaxf(pm[u], __shfl_xor(pm[u], 32));
+        }
+        if (wave < waves && (lane & 0x33) == 0) {
+#pragma unroll
+            for (int u = 0; u < XU; u++) wmax[wave * 32 + 4 * u + rr] = pm[u];
+        }
+        __syncthreads();
+        RowQuant rq[XU];
+#pragma unroll
+        for (int u = 0; u < XU; u++) {
+            float amax = 0.0f;
+            for (int w = 0; w < waves; w++) amax = fmaxf(amax, wmax[w * 32 + 4 * u + rr]);
+            rq[u] = row_quant(amax);
+        }
+        if (wave == 0 && (lane & 0x33) == 0) {
+#pragma unroll
+            for (int u = 0; u < XU; u++) {
+                xscale[4 * u + rr] = rq[u].s;
+                if (a.row_scale_out && blockIdx.x == 0 && 4 * u + rr < a.m) a.row_scale_out[4 * u + rr] = rq[u].s;
+            }
+        }
+        if (nkb <= KB_MAX) {
+#pragma unroll
+            for (int i = 0; i < KB_MAX; i++) {
+                if (i < nkb) {
+#pragma unroll
+                    for (int u = 0; u < XU; u++) {
+                        const u32x2 lo = quantize8_bf16(raw[i][u][0], rq[u]), hi = quantize8_bf16(raw[i][u][1], rq[u]);
+                        *reinterpret_cast<u32x4*>(xres + (size_t)((kb0 + i * waves) * XU + u) * 1024 + 16 * lane) =
+                            u32x4{lo.x, lo.y, hi.x, hi.y};
+                    }
+                }
+            }
+        } else {
+            for (int kb = kb0; kb < blocks; kb += waves)
+#pragma unroll
+                for (int u = 0; u < XU; u++) {
+                    const u32x4* src = chunk(a, kb, u);
+                    const u32x2 lo = quantize8_bf16(src[0], rq[u]), hi = quantize8_bf16(src[1], rq[u]);
+                    *reinterpret_cast<u32x4*>(xres + (size_t)(kb * XU + u) * 1024 + 16 * lane) = u32x4{lo.x, lo.y, hi.x, hi.y};
+                }
+        }
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // Persistent variant for shapes with many more tiles than CUs.  A workgroup walks a contiguous
 // run of tiles (persistent_tile_run) and every wave's ring simply continues across the
@@ -257,8 +374,14 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
 // (The reference's kernel is persistent for the same reason: skinny_gemm_kernel.cu:44-51.)
 // The reduction scratch is double-buffered by tile parity, which leaves one barrier per tile.
 // No cross-workgroup split-K in this variant.
-template <int MT, int RG, int XU, int DEPTH, bool NT, bool XRES>
-__global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_persistent_kernel(const StreamArgs a) {
+// QUANT: the activations arrive as bf16 (a.A16) and the workgroup quantises them itself (ActivationQuantizer); a separate
+// instantiation with room for 9 waves of 168 registers (the chunks it holds between its two steps), so that the
+// ordinary kernel keeps its registers.
+constexpr int kQuantThreads = 576;
+template <int MT, int RG, int XU, int DEPTH, bool NT, bool XRES, bool QUANT = false>
+__global__ void __launch_bounds__(QUANT ? kQuantThreads : lds_persistent_launch_bound(MT, RG))
+lds_gemm_persistent_kernel(const StreamArgs a) {
+    static_assert(!QUANT || XRES, "in-kernel quantisation writes the resident-activation layout");
     // XRES: [X blocks][XU KB] | [wave][DEPTH][RG*4 KB] | red;  else: [wave][DEPTH][(RG*4 + XU) KB] | red[2][FRAGS][wave][64]
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
 
@@ -294,6 +417,10 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     const uint8_t* my_ring = ring + x_bytes + (size_t)wave * (DEPTH * STAGE_BYTES);
     const unsigned my_ring_lds = lds_addr(my_ring);
     f32x4* red = reinterpret_cast<f32x4*>(ring + x_bytes + (size_t)waves * (DEPTH * STAGE_BYTES));
+    // bf16 activations quantised here (resident kernel only): the row scales live behind the reduction scratch
+    constexpr bool quant = QUANT;
+    float* xscale = reinterpret_cast<float*>(red + (size_t)2 * FRAGS * waves * 64);
+    const float* row_factors = quant ? xscale : nullptr;
 
     auto tile_origin = [&](int j, int& m0, int& n0) __attribute__((always_inline)) {  // j-th tile of this workgroup
         const int t = run.first + j;
@@ -351,13 +478,18 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
         if (waves == 1 && !epilogue_wave) {
 #pragma unroll
             for (int f = 0; f < FRAGS; f++)
-                store_fragment(a, acc[f / MT][f % MT], scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g);
+                store_fragment(a, acc[f / MT][f % MT], scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g, row_factors);
         } else {
             f32x4* buf = red + (size_t)(j & 1) * (FRAGS * waves * 64);
             if (wave < waves) {
 #pragma unroll
                 for (int f = 0; f < FRAGS; f++) buf[(f * waves + wave) * 64 + lane] = acc[f / MT][f % MT];
             }
+            // per-column factors of this tile, requested before the barrier: fetched when needed, their memory
+            // latency (a different line per tile) would be paid once per tile by the wave that stores
+            f32x4 colf[RG];
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) colf[rg] = col_scale_ahead(a, n0 + rg * 16 + 4 * g);
             __syncthreads();
             // without an epilogue wave the reducing wave rotates with the tile, so that the cost is
             // spread over the waves
@@ -370,7 +502,11 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
             for (int f = first; f < FRAGS; f += step) {
                 f32x4 v = buf[(f * waves) * 64 + lane];
                 for (int w = 1; w < waves; w++) v += buf[(f * waves + w) * 64 + lane];
-                store_fragment(a, v, scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g);
+                f32x4 cf = colf[0];    // colf[f / MT] without indexing registers by a run-time value
+#pragma unroll
+                for (int rg = 1; rg < RG; rg++)
+                    if (f / MT == rg) cf = colf[rg];
+                store_fragment(a, v, scale, m0 + (f % MT) * 16 + r, n0 + (f / MT) * 16 + 4 * g, row_factors, &cf);
             }
         }
 #pragma unroll
@@ -379,7 +515,9 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
             for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     };
 
-    if (XRES) {
+    ActivationQuantizer<QUANT ? XU : 1> aq;
+    if constexpr (quant) aq.load_and_max(a, blocks, waves, wave, lane);   // before the weight prologue: see ActivationQuantizer
+    if (XRES && !quant) {
         // K block kb of the activations is fetched by wave kb % waves; every wave then starts its
         // weight ring, waits for its own share (older than the ring's DMAs) and meets the others
         const unsigned x_lds = lds_addr(ring);
@@ -398,6 +536,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     }
 
     if (per_tile == 0) {  // more waves than K blocks: this wave only takes part in the reductions
+        if constexpr (quant) aq.finish(a, ring, reinterpret_cast<float*>(red), xscale, blocks, waves, wave, lane);
         if (XRES) {
             wait_vmcnt<0>();
             __syncthreads();
@@ -419,6 +558,8 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) issue(d);
         stamps.mark(1);
+        // the weights are on their way; meanwhile the workgroup quantises its copy of the activations
+        if constexpr (quant) aq.finish(a, ring, reinterpret_cast<float*>(red), xscale, blocks, waves, wave, lane);
         if (XRES) {
             wait_vmcnt_upto(DEPTH * PER_STAGE);   // this wave's activation blocks are older than its DEPTH stages
             __syncthreads();
@@ -441,6 +582,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
         drain_ring<0, DEPTH, PER_STAGE>(consume_and_close, i);
     } else {
         for (int i = 0; i < total; i++) issue(i);
+        if constexpr (quant) aq.finish(a, ring, reinterpret_cast<float*>(red), xscale, blocks, waves, wave, lane);
         wait_vmcnt<0>();
         if (XRES) __syncthreads();
         for (int i = 0; i < total; i++) {

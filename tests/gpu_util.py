@@ -31,10 +31,11 @@ def gemm_reference(oracle, a8, b8, scale, group=8, b_stride=None):
     return oracle.gemm_grouped(a8, b8, scale, group, b_stride=b_stride)
 
 
-def rowcol_reference(oracle, a8, b8, scale=1.0, row_scale=None, col_scale=None):
+def rowcol_reference(oracle, a8, b8, scale=1.0, row_scale=None, col_scale=None, model=False):
     """gemm_reference with the per-row / per-column factors of sg_skinny_gemm_rowcol: ((sum * scale) * row) * col,
-    each product rounded to fp32, one bf16 rounding."""
-    if a8.shape[1] >= MODEL_BELOW_K:
+    each product rounded to fp32, one bf16 rounding.  model=True takes the model of the instruction's summation
+    whatever k is (operands with a wide dynamic range inside a run of 8 k show the cut at long k as well)."""
+    if a8.shape[1] >= MODEL_BELOW_K and not model:
         return oracle.gemm_rowcol(a8, b8, scale, row_scale, col_scale)
     v = oracle.gemm_grouped(a8, b8, 1.0, 8, np.float32) * np.float32(scale)
     if row_scale is not None:
