@@ -143,7 +143,9 @@ typedef struct SgTuning {
                           stay resident in LDS; 2 = persistent K-split workgroups with resident activations
                           3 = the same with the activations in the wavefronts' registers (k = 256 * waves * 1, 2 or 4)
                           (all need persistent_wgs_per_cu >= 1, split_k = 1, m <= 16*m_blocks); + 4 = persistent
-                          workgroups get one extra wavefront that streams nothing and does every reduction and store */
+                          workgroups get one extra wavefront that streams nothing and does every reduction and store;
+                          8 (alone, with row_tiles = 2, m_blocks = 1, persistent_wgs_per_cu = 0) = 24-row tiles: the
+                          second 16-row fragment carries 8 weight rows (6144 rows = 256 tiles instead of 384) */
 } SgTuning;
 
 int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,

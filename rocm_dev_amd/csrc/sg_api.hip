@@ -220,12 +220,13 @@ static int attach_workspace(const Config& c, StreamArgs& a, size_t tiles, size_t
     return SG_SUCCESS;
 }
 
-static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out, hipStream_t stream) {
+static int prepare(const Config& c, StreamArgs& a, int stage_bytes_k, size_t* tiles_out, hipStream_t stream, int tile_rows = 0) {
     const int frags = c.rg * c.mt;
     if (c.waves < 1 || c.waves > 16 || c.depth < 1 || c.rg < 1 || c.mt < 1 || stage_bytes_k < 16) return SG_INVALID_CONFIG;
+    if (tile_rows <= 0) tile_rows = 16 * c.rg;
     a.waves = c.waves;
     a.split_k = c.split_k;
-    a.n_tiles = (a.n + 16 * c.rg - 1) / (16 * c.rg);
+    a.n_tiles = (a.n + tile_rows - 1) / tile_rows;
     a.m_tiles = (a.m + 16 * c.mt - 1) / (16 * c.mt);
     const int total_stages = a.k / stage_bytes_k > 0 ? a.k / stage_bytes_k : 1;
     if (c.split_k < 1 || c.split_k > total_stages) return SG_INVALID_CONFIG;
@@ -253,19 +254,22 @@ static int launch_stream(const Config& c, StreamArgs a, hipStream_t stream) {
 
 static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     if (a.k % 256 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    // wave_tiles bit 3: 24-row tiles (two fragments, the second half used), one workgroup per tile
+    const bool rows24 = (c.wavetile & 8) != 0;
+    if (rows24 && (c.rg != 2 || c.mt != 1 || c.persist != 0 || (c.wavetile & 7) != 0)) return SG_INVALID_CONFIG;
     size_t tiles;
-    if (int rc = prepare(c, a, 256, &tiles, stream)) return rc;
+    if (int rc = prepare(c, a, 256, &tiles, stream, rows24 ? 24 : 0)) return rc;
     // activation DMA instructions per stage: 4 rows each, rounded up to a compiled count
     int xu = 8;
     if (c.mt == 1) {
         const int need = (a.m + 3) / 4;
         xu = need <= 1 ? 1 : (need <= 2 ? 2 : 4);
     }
-    const size_t stage = (size_t)(c.rg * 4 + xu) * 1024;
+    const size_t stage = (size_t)((rows24 ? 6 : c.rg * 4) + xu) * 1024;
     // + 4 KB: lanes of activation rows that are not loaded read past the last slot
     size_t lds = (size_t)c.waves * c.depth * stage + 4096;
     unsigned grid = (unsigned)(tiles * c.split_k);
-    int mode = 0, extra_wave = 0;
+    int mode = rows24 ? 5 : 0, extra_wave = 0;
     if (a.A16 && !(c.persist > 0 && (c.wavetile & 3) == 2)) return SG_INVALID_CONFIG;
     if (c.wavetile == 1) {
         // whole activation matrix resident: one tile row of activations only, no K split
@@ -315,7 +319,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     }
     const unsigned threads = (unsigned)(c.waves + extra_wave) * 64;
     if (threads > 1024) return SG_TOO_MANY_WARPS;
-    if (mode == 0 || mode == 1 || mode == 3 || mode == 4) a.stamps = take_stamps(grid);
+    if (mode != 2) a.stamps = take_stamps(grid);
 #define SG_GO(MT, RG)                                                                                          \
     if (c.mt == MT && c.rg == RG)                                                                              \
         return SG_LDS_LAUNCHER(MT, RG)(xu, c.depth, c.nt, mode, a, grid, threads, lds, stream);
@@ -680,10 +684,23 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             c.rg = 1;
             c.waves = blocks >= 48 ? 2 : 1;
             c.depth = c.waves == 1 ? 8 : 4;
+            // between one and two 16-row tiles per CU half of the CUs stream twice what the others do (all
+            // workgroups are resident at once); 24-row tiles that give every CU one workgroup level that.  Measured
+            // on 6144 x 4096: level with 16-row tiles up to 8 activation rows (6.75 against 6.70 us - the launch is
+            // bound by its fixed costs and the stream rate, not by the imbalance), 3-5 % ahead at 9..16 rows
+            // (7.00 against 7.23-7.40 us), where the activation stage is shared by more weight rows.
+            const int tiles24 = (n + 23) / 24;
+            if (m > 8 && ((tiles24 + cu_count - 1) / cu_count) * 24 < ((tiles16 + cu_count - 1) / cu_count) * 16) {
+                c.rg = 2;
+                c.wavetile = 8;
+                c.waves = 2;
+                c.depth = 4;
+            }
         }
         const int xu = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
-        while (c.depth > 2 && ((c.depth - 1) * (c.rg * 4 + xu) > 63 ||
-                               (size_t)c.waves * c.depth * (c.rg * 4 + xu) * 1024 + 4096 > 159 * 1024))
+        const int w_instr = (c.wavetile & 8) ? 6 : c.rg * 4;
+        while (c.depth > 2 && ((c.depth - 1) * (w_instr + xu) > 63 ||
+                               (size_t)c.waves * c.depth * (w_instr + xu) * 1024 + 4096 > 159 * 1024))
             c.depth--;
         if (!c.persist && c.depth > blocks / c.waves && blocks / c.waves >= 2) c.depth = blocks / c.waves;
         if (c.depth == 5 || c.depth == 7) c.depth--;

@@ -110,14 +110,16 @@ __device__ __forceinline__ f32x4 col_scale_ahead(const StreamArgs& a, int n_idx)
     }
     return c;
 }
+// Columns from `n_limit` on belong to another tile (24-row tiles computed with two 16-row fragments) and are not written.
 __device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, float scale, int m_idx, int n_idx,
-                                               const float* lds_row_scale = nullptr, const f32x4* col_factors = nullptr) {
+                                               const float* lds_row_scale = nullptr, const f32x4* col_factors = nullptr,
+                                               int n_limit = 0x7fffffff) {
     // Pin the fragment before the lane-divergent exit below.  An MFMA needs every lane of the wave
     // (it reads all lanes' operand registers), but the compiler is free to sink the loads and the
     // MFMA that produce `v` into the region where only lanes with m_idx < m are active - it did so
     // with the 16x16x128 instruction - and the operand rows supplied by the masked lanes are then garbage.
     asm volatile("" : "+v"(v));
-    if (m_idx >= a.m) return;
+    if (m_idx >= a.m || n_idx >= n_limit) return;
     // scale, then the row factor, then the column factors: three separately rounded fp32 products
     v *= scale;
     if (lds_row_scale) v *= lds_row_scale[m_idx];
@@ -152,7 +154,7 @@ __device__ __forceinline__ void store_fragment(const StreamArgs& a, f32x4 v, flo
 
 template <int RG, int MT>
 __device__ __forceinline__ void finish_tile(const StreamArgs& a, f32x4 (&acc)[RG][MT], f32x4* red, unsigned* arrival_lds,
-                                            int tile_m, int tile_n, int split, int m0, int n0) {
+                                            int tile_m, int tile_n, int split, int m0, int n0, int n_limit = 0x7fffffff) {
     constexpr int FRAGS = RG * MT;
     const int lane = lane_id();
     const int wave = wave_id();
@@ -166,7 +168,7 @@ __device__ __forceinline__ void finish_tile(const StreamArgs& a, f32x4 (&acc)[RG
     auto finish = [&](int f, f32x4 v) __attribute__((always_inline)) {
         const int rg = f / MT, mt = f % MT;
         if (a.split_k == 1) {
-            store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g);
+            store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g, nullptr, nullptr, n_limit);
         } else {
             // agent-scope stores go through to memory, past this XCD's L2, so that a workgroup on
             // another XCD can read them without any cache-wide write-back or invalidate
@@ -214,7 +216,7 @@ __device__ __forceinline__ void finish_tile(const StreamArgs& a, f32x4 (&acc)[RG
             for (int e = 0; e < 4; e++) v[e] += __hip_atomic_load(q + e * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         const int rg = f / MT, mt = f % MT;
-        store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g);
+        store_fragment(a, v, scale, m0 + mt * 16 + r, n0 + rg * 16 + 4 * g, nullptr, nullptr, n_limit);
     }
     if (threadIdx.x == 0)  // ready for the next launch
         __hip_atomic_store(&a.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -11,10 +11,11 @@ namespace sg {
 
 template <int XU, int DEPTH, bool NT, int MODE>
 static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size_t lds, hipStream_t stream) {
-    constexpr int bound = MODE == 4 ? kQuantThreads : (MODE == 0 ? lds_launch_bound(SG_MT, SG_RG) : lds_persistent_launch_bound(SG_MT, SG_RG));
+    constexpr int bound = MODE == 4 ? kQuantThreads : ((MODE == 0 || MODE == 5) ? lds_launch_bound(SG_MT, SG_RG) : lds_persistent_launch_bound(SG_MT, SG_RG));
     if (threads > (unsigned)bound) return SG_INVALID_CONFIG;
     void (*kernel)(const StreamArgs) = nullptr;
     if constexpr (MODE == 4) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true, true>;
+    else if constexpr (MODE == 5) kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
     else if constexpr (MODE == 2) kernel = lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
     else if constexpr (MODE == 3) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
     else if constexpr (MODE == 1) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false>;
@@ -28,6 +29,13 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
 #define SG_CASE(XU_, DEPTH_)                                                                    \
     if (xu == XU_ && depth == DEPTH_) {                                                         \
         if constexpr (XU_ <= 4 * SG_MT && (SG_MT == 1 || XU_ > 4)) {                            \
+            if (mode == 5) { /* 24-row tiles: two fragments, six weight instructions per stage */ \
+                if constexpr (SG_MT == 1 && SG_RG == 2 && (DEPTH_ - 1) * (6 + XU_) <= 63)       \
+                    return nt ? launch_one<XU_, DEPTH_, true, 5>(a, grid, threads, lds, stream) \
+                              : launch_one<XU_, DEPTH_, false, 5>(a, grid, threads, lds, stream); \
+                else                                                                            \
+                    return SG_INVALID_CONFIG;                                                   \
+            }                                                                                   \
             if (mode == 4) { /* bf16 activations quantised in the kernel: one row tile per wave, two slots */ \
                 if constexpr (SG_RG == 1 && DEPTH_ == 2)                                        \
                     return nt ? launch_one<XU_, DEPTH_, true, 4>(a, grid, threads, lds, stream) \

@@ -134,12 +134,18 @@ constexpr int lds_launch_bound(int MT, int RG) { return RG * MT >= 8 ? 512 : 102
 constexpr int lds_persistent_launch_bound(int MT, int RG) { return RG * MT >= 4 ? 512 : 1024; }
 
 // XU = activation DMA instructions per stage (4 rows each): ceil(min(m, 16*MT) / 4)
-template <int MT, int RG, int XU, int DEPTH, bool NT>
+// HALF2 (RG == 2 only): 24-row tiles - the second 16-row fragment holds 8 weight rows, its other 8 are never fetched
+// (the MFMA reads whatever lies there) and never stored.  6144 rows are 256 tiles of 24 where they are 384 of 16: one
+// workgroup per CU instead of one and a half.
+template <int MT, int RG, int XU, int DEPTH, bool NT, bool HALF2 = false>
 __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
     __shared__ unsigned arrival;
 
-    constexpr int PER_STAGE = RG * 4 + XU;         // DMA instructions per stage
+    static_assert(!HALF2 || RG == 2, "24-row tiles are two fragments");
+    constexpr int W_INSTR = HALF2 ? 6 : RG * 4;    // weight DMA instructions per stage (4 rows each)
+    constexpr int TILE_ROWS = HALF2 ? 24 : 16 * RG;
+    constexpr int PER_STAGE = W_INSTR + XU;        // DMA instructions per stage
     constexpr int STAGE_BYTES = PER_STAGE * 1024;
     static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
     static_assert(XU <= 4 * MT, "more activation rows than the tile has");
@@ -152,7 +158,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
 
     int tile_n, split, tile_m;
     decode_tile(a, xcd_order((int)blockIdx.x, (int)gridDim.x), tile_n, split, tile_m);
-    const int n0 = tile_n * (16 * RG);
+    const int n0 = tile_n * TILE_ROWS;
     const int m0 = tile_m * (16 * MT);
 
     // K range of this workgroup in 256-byte blocks; the last split takes the remainder
@@ -199,11 +205,12 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
         for (int rg = 0; rg < RG; rg++)
 #pragma unroll
             for (int u = 0; u < 4; u++) {
+                if (rg * 4 + u >= W_INSTR) continue;
                 if (NT) dma_1kb_stream_at(w_base + koff, woff[rg][u], slot + (rg * 4 + u) * 1024);
                 else dma_1kb_at(w_base + koff, woff[rg][u], slot + (rg * 4 + u) * 1024);
             }
 #pragma unroll
-        for (int u = 0; u < XU; u++) dma_1kb_at(x_base + koff, xoff[u], slot + (RG * 4 + u) * 1024);
+        for (int u = 0; u < XU; u++) dma_1kb_at(x_base + koff, xoff[u], slot + (W_INSTR + u) * 1024);
     };
 
     f32x4 acc[RG][MT];
@@ -214,7 +221,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
 
     auto consume = [&](int i) __attribute__((always_inline)) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
-        mma_block_256<MT, RG>(slot, slot + RG * 4096, acc);
+        mma_block_256<MT, RG>(slot, slot + W_INSTR * 1024, acc);
     };
 
     if (mine >= DEPTH) {
@@ -246,7 +253,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     stamps.mark(3);
     __syncthreads();
-    finish_tile<RG, MT>(a, acc, reinterpret_cast<f32x4*>(ring), &arrival, tile_m, tile_n, split, m0, n0);
+    finish_tile<RG, MT>(a, acc, reinterpret_cast<f32x4*>(ring), &arrival, tile_m, tile_n, split, m0, n0, n0 + TILE_ROWS);
     stamps.end(a);
 }
 

@@ -31,6 +31,15 @@ def expect_lds(m, n, k, r):
     blocks = k // 256
     if not (1 <= waves <= 16 and depth >= 1 and rg >= 1 and mt in (1, 2) and 1 <= sk <= blocks):
         return INVALID
+    if wt & 8:                                            # 24-row tiles: two fragments, six weight instructions per stage
+        if rg != 2 or mt != 1 or persist != 0 or wt != 8:
+            return INVALID
+        per_stage = 6 + activation_instructions(m, 1)
+        if waves * depth * per_stage * 1024 + 4096 > LDS_USABLE:
+            return INVALID
+        if waves * 64 > 1024:
+            return TOO_MANY_WARPS
+        return OK if depth in (2, 3, 4, 6, 8) and (depth - 1) * per_stage <= VMCNT_MAX else INVALID
     xu = activation_instructions(m, mt)
     m_tiles = -(-m // (16 * mt))
     frags = rg * mt

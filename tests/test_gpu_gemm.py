@@ -157,6 +157,40 @@ def test_lds_ring_engine(sg, oracle, cfg, shape):
     assert np.array_equal(bits(D2), got)
 
 
+@pytest.mark.parametrize("cfg", [(1, 1, 8), (1, 2, 4), (2, 1, 4), (1, 4, 2), (3, 2, 3), (1, 1, 6)])
+@pytest.mark.parametrize("shape", [(8, 6144, 4096), (5, 130, 512), (16, 1000, 1024), (8, 50, 256), (1, 24, 768), (13, 6144, 1024),
+                                   (32, 96, 512)])
+def test_lds_ring_24_row_tiles(sg, oracle, cfg, shape):
+    """24-row tiles: two 16-row fragments of which the second carries 8 weight rows; its other 8 rows are never fetched
+    and never stored (they belong to the next tile).  n a multiple of 24, ragged n (last tile of 10, of 16, of 2 rows),
+    one tile only, K split across workgroups and waves.  m above 16 has no such kernel."""
+    split_k, waves, depth = cfg
+    m, n, k = shape
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=24)
+    ref = gemm_reference(oracle, a8, b8, scale)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kw = dict(engine=2, split_k=split_k, waves=waves, row_tiles=2, m_blocks=1, depth=depth, wave_tiles=8)
+    rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
+    torch.cuda.synchronize()
+    want = expect_lds(m, n, k, record(2, split_k, waves, 2, 1, depth, 4, 1, 0, 8)) if m <= 16 else 6
+    if m > 16:
+        kw["m_blocks"] = 2
+        rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
+    assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
+    if rc != 0:
+        pytest.skip("the configuration does not fit this shape, and the library says so")
+    got = bits(D)
+    assert not np.isnan(oracle.bf16_to_f32(got)).any(), "an output was left unwritten"
+    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    # 16-row tiles with the same K split sum the same products in the same order: identical bits
+    D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    kw.update(row_tiles=1, wave_tiles=0)
+    if sg.skinny_gemm_tuned(A, B, D2, S, **kw) == 0:
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(D2), got)
+
+
 PERSISTENT_CONFIGS = [
     # waves, row_tiles, depth, persistent workgroups per CU
     (1, 1, 4, 1),

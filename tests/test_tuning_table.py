@@ -120,10 +120,10 @@ def test_search_space_respects_the_fit_rules():
                 assert autotune.lds_ring_fits(m, k, r)
                 mode = r["wave_tiles"] & 3
                 xu = autotune._activation_instructions(m, r["m_blocks"])
-                per_stage = 4 * r["row_tiles"] + (0 if mode else xu)
+                per_stage = (6 if r["wave_tiles"] & 8 else 4 * r["row_tiles"]) + (0 if mode else xu)
                 assert r["waves"] * r["depth"] * per_stage * 1024 < autotune.LDS_BYTES
                 assert (r["depth"] - 1) * per_stage <= 63
-                if r["persistent_wgs_per_cu"] or r["wave_tiles"]:
+                if r["persistent_wgs_per_cu"] or r["wave_tiles"] & 7:     # (24-row tiles, bit 3, may split K)
                     assert r["split_k"] == 1
     # the library's own choices for the benchmark shapes are inside the space
     import rocm_dev_amd as sg
