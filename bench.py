@@ -66,6 +66,11 @@ def main():
                          "on cold weights through the library's choice and three times through the one-wave-workgroup kernel "
                          "it replaced, after three 256 MiB copies of known traffic, and exit (for L2 / HBM traffic counter runs; "
                          "prints no JSON line)")
+    ap.add_argument("--ring-ab", action="store_true",
+                    help="only compare the producer/consumer ring (sg_skinny_gemm with producers > 0, best record of a sweep "
+                         "over producers x consumers x b_lanes x qsize) with the library's own choice on the four projection "
+                         "shapes at M = 8 and 32, cold weights; then launch each winner and each own choice ten times eagerly "
+                         "(for a kernel trace); prints a table, no JSON line")
     ap.add_argument("--stamps", action="store_true",
                     help="only run the decode GEMMs (four projection shapes at M = --m) back to back from a HIP graph with "
                          "the library's per-workgroup time stamps switched on, and print where a launch period goes "
@@ -84,6 +89,73 @@ def main():
     torch.manual_seed(0)
     if lib.sg_init() != 0:
         sys.exit("bench.py: sg_init failed")
+
+    if args.ring_ab:
+        import itertools
+        from rocm_dev_amd import autotune, synth
+        side = torch.cuda.Stream()
+
+        def time_us(fn, reps=20, replays=7):
+            with torch.cuda.stream(side):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    st = torch.cuda.current_stream().cuda_stream
+                    for i in range(reps):
+                        if fn(i, st) != 0:
+                            return None
+                ts = []
+                for r in range(replays + 2):
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a.record()
+                    g.replay()
+                    b.record()
+                    torch.cuda.synchronize()
+                    if r >= 2:
+                        ts.append(a.elapsed_time(b) * 1e3 / reps)
+            return sorted(ts)[len(ts) // 2]
+
+        print("producer/consumer ring against the library's own choice; us per launch, median of 7 graph replays of 20 "
+              "launches on cold weights")
+        print("| shape | M | own choice (us) | best ring record (us) | ring / own | ring record: A producers, B producers, "
+              "consumers, b_lanes, qsize |")
+        print("|---|---|---|---|---|---|")
+        eager = []
+        for name, (n, k) in SHAPES.items():
+            copies = max(3, int(COLD_BYTES // (n * k)) + 1)
+            wb = [synth.quantize_tensor(synth.normal_f32((n, k), c, 2))[0] for c in range(copies)]
+            one = torch.ones(1, device="cuda")
+            for m in (8, 32):
+                a8 = synth.quantize_tensor(synth.normal_f32((m, k), 0, 1))[0]
+                d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+                op_m = 8 if m <= 8 else (16 if m <= 16 else 32)
+                ops = 256 // (512 // op_m)
+                own = time_us(lambda i, st: lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(),
+                                                                    one.data_ptr(), m, n, k, k, st))
+                best = (1e30, None)
+                for ap_, bp, cons, bl, qs in itertools.product((1, 2), (2, 4, 6, 8), (1, 2, 3, 4), (1, 2, 4), (2, 3, 4, 6, 8)):
+                    if ap_ + bp + cons > 16 or qs < max(ap_, bp // bl, cons) or not autotune.pc_ring_fits(m, k, ap_, bp, cons, bl, qs):
+                        continue
+                    t = time_us(lambda i, st: lib.sg_skinny_gemm(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(),
+                                                                 one.data_ptr(), m, n, k, k, 1, ap_, bp, cons, bl, qs, op_m, ops, st),
+                                reps=10, replays=3)
+                    if t is not None and t < best[0]:
+                        best = (t, (ap_, bp, cons, bl, qs))
+                ap_, bp, cons, bl, qs = best[1]
+                ring = time_us(lambda i, st: lib.sg_skinny_gemm(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(),
+                                                                one.data_ptr(), m, n, k, k, 1, ap_, bp, cons, bl, qs, op_m, ops, st))
+                print("| %s %d x %d | %d | %.2f | %.2f | %.2f | %d, %d, %d, %d, %d |"
+                      % (name, n, k, m, own, ring, ring / own, ap_, bp, cons, bl, qs), flush=True)
+                eager.append((name, m, a8, d, best[1], op_m, ops))
+            # ten eager launches of each (for rocprofv3 --kernel-trace --stats): the own choice, then the ring
+            for (nm, m, a8, d, rec, op_m, ops) in [e for e in eager if e[0] == name]:
+                for i in range(10):
+                    lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, None)
+                for i in range(10):
+                    lib.sg_skinny_gemm(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, 1,
+                                       rec[0], rec[1], rec[2], rec[3], rec[4], op_m, ops, None)
+                torch.cuda.synchronize()
+            del wb
+        return
 
     if args.stamps:
         import numpy as np

@@ -112,7 +112,7 @@ def mid_fits(k, r):
     if (r["depth"] * bn + dx * bm) * 128 + (16 if r["split_k"] > 1 else 0) > LDS_BYTES:
         return False
     blocks = k // 128
-    return r["split_k"] == 1 or blocks // r["split_k"] >= 32
+    return r["split_k"] == 1 or blocks // r["split_k"] >= 8
 
 
 def search_space(m, n, k):
@@ -120,7 +120,7 @@ def search_space(m, n, k):
     authority: a candidate it has no kernel for comes back SG_INVALID_CONFIG and is skipped."""
     out = []
     if m > 32 and k % 128 == 0:
-        for waves, rt, mb, depth, dx, sk in itertools.product((4, 8, 14), (2, 4), (2, 4, 8), (2, 3, 4, 6), (0, 2, 3), (1, 2, 4)):
+        for waves, rt, mb, depth, dx, sk in itertools.product((4, 8, 14), (2, 4), (2, 4, 8), (2, 3, 4, 6), (0, 2, 3), (1, 2, 3, 4, 5, 6, 8)):
             if dx and dx >= depth:
                 continue
             if waves == 14 and rt != 2:             # 224-row tiles: seven waves along n, two fragments each
