@@ -37,14 +37,40 @@ def project_dir(name):
     return d
 
 
-def compile_main(project, c_file):
+def _sources(project):
+    """Everything a main of `project` is compiled from: its own directory, the shared harness header, the library's
+    kernel sources and the oracle's C file."""
+    root = os.path.dirname(os.path.dirname(HERE))
+    dirs = [project_dir(project), os.path.join(root, "rocm_dev_amd", "csrc"), os.path.join(root, "oracle")]
+    files = [os.path.join(HERE, "projects", "common.cuh")]
+    for d in dirs:
+        files += [os.path.join(d, f) for f in os.listdir(d) if f.endswith((".cu", ".cuh", ".h", ".hip", ".c"))]
+    return files
+
+
+def compile_main(project, c_file, force=False):
+    """hipcc <project>/<c_file> -> build/<project>.<stem>.out; an executable newer than all of its sources is kept
+    (the mains are compiled ahead of a GPU run, which then only executes them)."""
     os.makedirs(BUILD, exist_ok=True)
-    out = os.path.join(BUILD, c_file.split(".")[0] + ".out")
+    out = os.path.join(BUILD, "%s.%s.out" % (project, c_file.split(".")[0]))
+    if not force and os.path.exists(out) and os.path.getmtime(out) >= max(os.path.getmtime(f) for f in _sources(project)):
+        return out
     res = subprocess.run(["hipcc"] + HIPCC_FLAGS + [os.path.join(project_dir(project), c_file), "-o", out],
                          capture_output=True, text=True)
     if res.returncode != 0:
         raise subprocess.CalledProcessError(res.returncode, "hipcc", stderr=res.stderr[-2000:])
     return out
+
+
+PROJECTS = ("skinny_gemm", "async_gemm_sparse", "async_gemm_blanes", "async_gemm_16x16x64", "tiled_sum_reduce",
+            "tiled_sum_reduce_async")
+
+
+def compile_all(jobs=6):
+    """Compiles test.cu and bench.cu of every project (what a build step runs ahead of the GPU tests)."""
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(jobs) as pool:
+        return list(pool.map(lambda pf: compile_main(*pf), [(p, f) for p in PROJECTS for f in ("test.cu", "bench.cu")]))
 
 
 def run_main(exe, arguments, timeout=None):

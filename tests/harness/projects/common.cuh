@@ -37,3 +37,19 @@ inline void random_host_fp8(std::vector<fp8>& x, size_t n) {
     }
 }
 inline float random_host_scale() { return static_cast<float>(rand()) / static_cast<float>(RAND_MAX) - 0.5f; }
+
+// U[-1, 1) floats, as the reference's random_host_tensor<float> (common.cuh:86-95)
+inline void random_host_f32(std::vector<float>& x, size_t n) {
+    x.resize(n);
+    for (size_t i = 0; i < n; i++) x[i] = 2 * (static_cast<float>(rand()) / static_cast<float>(RAND_MAX) - 0.5f);
+}
+
+// The role of the reference's flush_device_cache (common.cuh:141-158: a kernel that sweeps an L2-sized buffer):
+// here a fill of 640 MB, more than twice the 256 MB memory-side cache, so the next launch finds nothing of its
+// operands in any cache.  The buffer is allocated once.
+inline void flush_device_cache() {
+    static void* sweep = nullptr;
+    const size_t bytes = (size_t)640 << 20;
+    if (!sweep) HIP_CHECK(hipMalloc(&sweep, bytes));
+    HIP_CHECK(hipMemsetAsync(sweep, 0, bytes, 0));
+}

@@ -51,9 +51,13 @@ def test_core_rewrite_touches_only_define_lines(tmp_path):
 
 
 def test_mains_compile_for_gfx950():
-    """Single translation unit, kernels included as headers, exactly one instantiation."""
-    for f in ("test.cu", "bench.cu"):
-        assert os.path.exists(driver.compile_main("skinny_gemm", f))
+    """Single translation unit per main, kernels included as source, for every project the reference's drivers name
+    with -p: skinny_gemm, the three async_gemm_* ancestors, tiled_sum_reduce and its _async variant."""
+    for exe in driver.compile_all():
+        assert os.path.exists(exe)
+    for p in driver.PROJECTS:
+        for f in ("test.cu", "bench.cu"):
+            assert os.path.exists(os.path.join(ROOT, "tests", "harness", "projects", p, f)), (p, f)
 
 
 @pytest.mark.gpu
@@ -62,3 +66,23 @@ def test_protocol_end_to_end():
     worst = float(data["max_deltas"].split()[0])
     assert worst <= 0.05                      # bf16 outputs of magnitude ~1: one ulp is 2^-8
     assert 0.5 < data["median"] < 200.0       # microseconds per GEMM
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("project", ["tiled_sum_reduce", "tiled_sum_reduce_async"])
+def test_protocol_tiled_sum_reduce(project):
+    """argv = b m n (tiled_sum_reduce/test.cu:28-33); the batch sum is bit-identical to the host loop, so both deltas are 0."""
+    data = driver.main(["bench", "-p", project, "-a", "5 256 2050", "-t", "2"])
+    assert data["max_deltas"].split()[0] == "0.0000" and data["sum_deltas"].split()[0] == "0.0000"
+    assert 0.5 < data["median"] < 500.0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("project,args", [("async_gemm_sparse", "8 512 1024"), ("async_gemm_blanes", "16 1000 2048"),
+                                          ("async_gemm_16x16x64", "24 256 512")])
+def test_protocol_async_gemm(project, args):
+    """argv = m n k (async_gemm_sparse/test.cu:44-48); fp32 output of U[-1, 1) operands against the host's sequential
+    fp32 sum: what is left is summation order and the instruction's in-run cut, far below 1e-2 at these sizes."""
+    data = driver.main(["bench", "-p", project, "-a", args, "-t", "2"])
+    assert float(data["max_deltas"].split()[0]) <= 1e-2
+    assert 0.5 < data["median"] < 500.0
