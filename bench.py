@@ -32,7 +32,7 @@ COLD_BYTES = 640e6          # per shape: distinct weight bytes cycled through (>
 # HBM bytes per launch of the dominant kernel (gate_up, M = 8), measured off-line with two
 # rocprofv3 --pmc runs (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0, factors from a 256 MiB copy);
 # the runs and their arithmetic are in profiles/dense_gemm_decode_step_m8_pmc_traffic.md
-RECORDED_TRAFFIC = {"bytes": 118372433, "source": "profiles/dense_gemm_decode_step_m8_pmc_traffic.md",
+RECORDED_TRAFFIC = {"bytes": 118379600, "source": "profiles/dense_gemm_decode_step_m8_pmc_traffic.md",
                     # the kernel configuration the counters were read on; another configuration reports no traffic
                     "tuning": {"engine": 2, "waves": 8, "row_tiles": 1, "depth": 2, "persistent_wgs_per_cu": 1, "wave_tiles": 6}}
 
@@ -48,6 +48,11 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--m", type=int, default=8, help="activation rows of the timed step")
+    ap.add_argument("--random-codes", action="store_true",
+                    help="fill the operands with uniformly random E4M3 codes from torch's generator (one kernel per buffer) "
+                         "instead of the seeded N(0,1) recipe (dozens of elementwise kernels per buffer): for profiler runs "
+                         "that serialise every dispatch; timings of such a run are not the benchmark's")
+    ap.add_argument("--replays", type=int, default=31, help="timed regions per measurement (the median is reported)")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-warm", action="store_true", help="skip the cache-resident (same weight buffer) timings")
@@ -66,6 +71,15 @@ def main():
                          "on cold weights through the library's choice and three times through the one-wave-workgroup kernel "
                          "it replaced, after three 256 MiB copies of known traffic, and exit (for L2 / HBM traffic counter runs; "
                          "prints no JSON line)")
+    ap.add_argument("--n-sweep", action="store_true",
+                    help="only run 8 x N x 4096 for N = 4096 ... 57344 (1 ... 14 sixteen-row tiles per CU): the library's own "
+                         "choice, the per-tile kernel (one wave, eight slots) and the read-only streaming yardstick "
+                         "(sg_debug_read_stream), graph-timed on cold weights and then ten eager launches each (for a kernel "
+                         "trace); prints a table and the straight-line fit fixed + bytes / rate, no JSON line")
+    ap.add_argument("--codec-counters", action="store_true",
+                    help="only launch the 8192 x 8192 row codec (encode, decode, reduce of 8), the fp32 batch sum "
+                         "(8 x 1024 x 8192) and the read-only streaming yardstick on 28672 x 4096 three times each, eagerly, "
+                         "after three 256 MiB copies of known traffic, and exit (for kernel traces and HBM-traffic counters)")
     ap.add_argument("--ring-ab", action="store_true",
                     help="only compare the producer/consumer ring (sg_skinny_gemm with producers > 0, best record of a sweep "
                          "over producers x consumers x b_lanes x qsize) with the library's own choice on the four projection "
@@ -89,6 +103,101 @@ def main():
     torch.manual_seed(0)
     if lib.sg_init() != 0:
         sys.exit("bench.py: sg_init failed")
+
+    if args.n_sweep:
+        import ctypes
+        import numpy as np
+        from rocm_dev_amd import synth
+        side = torch.cuda.Stream()
+        m, k = 8, 4096
+        one = torch.ones(1, device="cuda")
+        a8 = synth.quantize_tensor(synth.normal_f32((m, k), 0, 1))[0]
+        per_tile = sg.SgTuning(2, 1, 1, 1, 1, 8, 4, 1, 0, 0)
+
+        def graph_us(fn, reps=24, replays=9):
+            with torch.cuda.stream(side):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=side):
+                    st = torch.cuda.current_stream().cuda_stream
+                    for i in range(reps):
+                        if fn(i, st) != 0:
+                            raise RuntimeError("launch failed")
+                ts = []
+                for r in range(replays + 3):
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a.record()
+                    g.replay()
+                    b.record()
+                    torch.cuda.synchronize()
+                    if r >= 3:
+                        ts.append(a.elapsed_time(b) * 1e3 / reps)
+            return sorted(ts)[len(ts) // 2]
+
+        print("8 x N x 4096, cold weights, us per launch (median of 9 graph replays of 24 launches)")
+        print("| N | tiles per CU | MB per launch | own choice | per-tile kernel (1 wave x 8 slots) | read-only yardstick |")
+        print("|---|---|---|---|---|---|")
+        xs, own_t, tile_t, read_t = [], [], [], []
+        for n in (4096, 8192, 12288, 16384, 20480, 24576, 28672, 32768, 40960, 57344):
+            copies = max(3, int(COLD_BYTES // (n * k)) + 1)
+            wb = [synth.quantize_tensor(synth.normal_f32((n, k), c, 2))[0] for c in range(copies)]
+            d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+            fns = (lambda i, st: lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, st),
+                   lambda i, st: lib.sg_skinny_gemm_tuned(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k,
+                                                          ctypes.byref(per_tile), st),
+                   lambda i, st: lib.sg_debug_read_stream(wb[i % copies].data_ptr(), n, k, k, st))
+            t = [graph_us(f) for f in fns]
+            mb = gemm_bytes(m, n, k) / 1e6
+            print("| %d | %.1f | %.1f | %.2f | %.2f | %.2f |" % (n, n / 16 / 256, mb, t[0], t[1], t[2]), flush=True)
+            xs.append(mb); own_t.append(t[0]); tile_t.append(t[1]); read_t.append(t[2])
+            for f in fns:                      # ten eager launches each, for rocprofv3 --kernel-trace
+                for i in range(10):
+                    f(i, None)
+                torch.cuda.synchronize()
+            del wb
+        for label, ys in (("own choice", own_t), ("per-tile kernel", tile_t), ("read-only yardstick", read_t)):
+            slope, fixed = np.polyfit(np.array(xs), np.array(ys), 1)
+            print("%s: %.2f us fixed + bytes / %.2f TB/s (least squares over the ten sizes)" % (label, fixed, 1.0 / slope))
+        return
+
+    if args.codec_counters:
+        from rocm_dev_amd import synth
+        src = torch.empty(256 << 20, device="cuda", dtype=torch.uint8)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        rows = cols = 8192
+        xs = [synth.normal_f32((rows, cols), i, 3).bfloat16() for i in range(3)]
+        q8 = torch.empty((8, rows, cols), device="cuda", dtype=torch.uint8)
+        s8 = torch.empty((8, rows), device="cuda", dtype=torch.float32)
+        y = torch.empty((rows, cols), device="cuda", dtype=torch.bfloat16)
+        for i in range(8):
+            lib.sg_fp8_encode_rows(xs[i % 3].data_ptr(), q8[i].data_ptr(), s8[i].data_ptr(), rows, cols, None)
+        torch.cuda.synchronize()
+        for i in range(3):
+            lib.sg_fp8_encode_rows(xs[i].data_ptr(), q8[i].data_ptr(), s8[i].data_ptr(), rows, cols, None)
+        torch.cuda.synchronize()
+        for i in range(3):
+            lib.sg_fp8_decode_rows(q8[3 + i].data_ptr(), s8[3 + i].data_ptr(), y.data_ptr(), rows, cols, None)
+        torch.cuda.synchronize()
+        for i in range(3):
+            lib.sg_fp8_reduce_rows(q8.data_ptr(), s8.data_ptr(), y.data_ptr(), 8, rows * cols, rows, cols, None)
+        torch.cuda.synchronize()
+        del xs, q8, s8, y
+        tb, tm, tn = 8, 1024, 8192
+        ta = synth.normal_f32((tb, tm, tn), 0, 4)
+        tbb = synth.normal_f32((tb, tm, tn), 0, 5)
+        td = torch.empty((tm, tn), device="cuda", dtype=torch.float32)
+        for i in range(3):
+            lib.sg_tiled_sum_reduce(ta.data_ptr(), tbb.data_ptr(), td.data_ptr(), tb, tm, tn, None)
+        torch.cuda.synchronize()
+        del ta, tbb, td
+        n, k = SHAPES["gate_up"]
+        wb = [synth.quantize_tensor(synth.normal_f32((n, k), c, 2))[0] for c in range(6)]
+        for i in range(6):
+            lib.sg_debug_read_stream(wb[i].data_ptr(), n, k, k, None)
+        torch.cuda.synchronize()
+        return
 
     if args.ring_ab:
         import itertools
@@ -307,6 +416,18 @@ def main():
         """Per-tensor scale absmax/448 and OCP E4M3 codes (round to nearest even)."""
         return synth.quantize_tensor(x)
 
+    if args.random_codes:
+        class _Codes:   # stands in for the seeded generator: same shapes, arbitrary finite codes
+            @staticmethod
+            def normal_f32(shape, seed, stream_id):
+                return torch.randint(0, 0x7E, shape, device="cuda", dtype=torch.uint8)
+
+            @staticmethod
+            def quantize_tensor(x):
+                return x, torch.full((), 1e-4, device="cuda")
+        synth = _Codes
+        quantize = _Codes.quantize_tensor
+
     # ---- synthetic operands, resident in HBM: the seeded counter generator of rocm_dev_amd.synth ------------
     # (seed 0, stream 1) = activations, (seed c, stream 2) = copy c of a weight matrix: copy 0 is the configuration's
     # own "N(0,1), seed 0" recipe, the further copies only exist so that the weights are cold
@@ -347,7 +468,7 @@ def main():
         for name in order:
             launch(name, args.m, i, stream)
 
-    REPLAYS = 31
+    REPLAYS = max(1, args.replays)
 
     def stats(samples):
         """median, 10th / 90th percentile and minimum of a list of timings"""

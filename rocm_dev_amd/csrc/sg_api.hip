@@ -12,6 +12,7 @@
 #include "sg_stream_kernel.h"
 #include "sg_ring_kernel.h"
 #include "sg_sparse_kernel.h"
+#include "sg_debug_kernel.h"
 #include <string>
 
 namespace sg {
@@ -891,6 +892,17 @@ int sg_debug_stamps(unsigned long long* device_buffer, size_t n_words) {
     g_stamp_words = device_buffer ? n_words : 0;
     g_stamp_cursor = 0;
     return SG_SUCCESS;
+}
+
+int sg_debug_read_stream(const uint8_t* B, int n, int k, int b_stride, void* stream) {
+    if (!B || n <= 0 || k <= 0 || k % 256 != 0 || b_stride < k || (b_stride & 15) || (reinterpret_cast<uintptr_t>(B) & 15u))
+        return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    const int tiles = (n + 15) / 16;
+    const unsigned grid = (unsigned)(tiles < dev->cu_count ? tiles : dev->cu_count);
+    read_stream_kernel<<<dim3(grid), dim3(512), 8 * 2 * 4096, static_cast<hipStream_t>(stream)>>>(B, n, k, b_stride, nullptr);
+    return report_hip("read_stream_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }
 
 int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,
