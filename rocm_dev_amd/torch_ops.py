@@ -1,0 +1,101 @@
+"""The library's GEMMs and codec as registered torch operators (namespace ``sgemm``).
+
+The reference builds a pybind extension (skinny_gemm/setup.py:11-20) whose class method fills a caller-provided
+tensor (skinny_gemm_binding.cu:16-100) - kept here as ``rocm_dev_amd.HFRK_skinny_gemm``.  These operators are the
+functional form ``torch.library`` and ``torch.compile`` understand: they allocate and return their result, declare
+their output shapes through fake (meta) implementations, and launch on torch's current stream through the same C ABI.
+
+    import rocm_dev_amd.torch_ops                      # registers torch.ops.sgemm.*
+    D = torch.ops.sgemm.skinny_gemm(A_fp8, W_fp8, scale)                    # [m, n] bf16
+    D = torch.ops.sgemm.skinny_gemm_rowcol(A_fp8, W_fp8, scale, row_scales, col_scales)
+    D = torch.ops.sgemm.skinny_gemm_bf16act(X_bf16, W_fp8, scale, col_scales)
+    Q, s = torch.ops.sgemm.fp8_encode_rows(X_bf16)
+    Y = torch.ops.sgemm.fp8_decode_rows(Q, s)
+    D = torch.ops.sgemm.sparse24_gemm(A_fp8, vals, meta, scale)
+
+FP8 operands are uint8 or float8_e4m3fn tensors holding OCP E4M3 codes; weights are [n, k] with k contiguous.
+"""
+from typing import Optional, Tuple
+
+import torch
+
+from . import api
+
+
+def _bytes(t):
+    return t.view(torch.uint8) if t.dtype == torch.float8_e4m3fn else t
+
+
+@torch.library.custom_op("sgemm::skinny_gemm", mutates_args=())
+def skinny_gemm(A: torch.Tensor, B: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    D = torch.empty((A.shape[0], B.shape[0]), dtype=torch.bfloat16, device=A.device)
+    api.skinny_gemm_fastpath(_bytes(A), _bytes(B), D, scale, check=True)
+    return D
+
+
+@skinny_gemm.register_fake
+def _(A, B, scale):
+    return A.new_empty((A.shape[0], B.shape[0]), dtype=torch.bfloat16)
+
+
+@torch.library.custom_op("sgemm::skinny_gemm_rowcol", mutates_args=())
+def skinny_gemm_rowcol(A: torch.Tensor, B: torch.Tensor, scale: Optional[torch.Tensor] = None,
+                       row_scales: Optional[torch.Tensor] = None, col_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
+    D = torch.empty((A.shape[0], B.shape[0]), dtype=torch.bfloat16, device=A.device)
+    api.skinny_gemm_rowcol(_bytes(A), _bytes(B), D, scale, row_scales, col_scales, check=True)
+    return D
+
+
+@skinny_gemm_rowcol.register_fake
+def _(A, B, scale=None, row_scales=None, col_scales=None):
+    return A.new_empty((A.shape[0], B.shape[0]), dtype=torch.bfloat16)
+
+
+@torch.library.custom_op("sgemm::skinny_gemm_bf16act", mutates_args=())
+def skinny_gemm_bf16act(X: torch.Tensor, B: torch.Tensor, scale: Optional[torch.Tensor] = None,
+                        col_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
+    D = torch.empty((X.shape[0], B.shape[0]), dtype=torch.bfloat16, device=X.device)
+    api.skinny_gemm_bf16act(X, _bytes(B), D, scale, col_scales, check=True)
+    return D
+
+
+@skinny_gemm_bf16act.register_fake
+def _(X, B, scale=None, col_scales=None):
+    return X.new_empty((X.shape[0], B.shape[0]), dtype=torch.bfloat16)
+
+
+@torch.library.custom_op("sgemm::fp8_encode_rows", mutates_args=())
+def fp8_encode_rows(X: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    Q = torch.empty(X.shape, dtype=torch.uint8, device=X.device)
+    s = torch.empty((X.shape[0],), dtype=torch.float32, device=X.device)
+    api.fp8_encode_rows(X, Q, s, check=True)
+    return Q, s
+
+
+@fp8_encode_rows.register_fake
+def _(X):
+    return X.new_empty(X.shape, dtype=torch.uint8), X.new_empty((X.shape[0],), dtype=torch.float32)
+
+
+@torch.library.custom_op("sgemm::fp8_decode_rows", mutates_args=())
+def fp8_decode_rows(Q: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    Y = torch.empty(Q.shape, dtype=torch.bfloat16, device=Q.device)
+    api.fp8_decode_rows(_bytes(Q), scales, Y, check=True)
+    return Y
+
+
+@fp8_decode_rows.register_fake
+def _(Q, scales):
+    return Q.new_empty(Q.shape, dtype=torch.bfloat16)
+
+
+@torch.library.custom_op("sgemm::sparse24_gemm", mutates_args=())
+def sparse24_gemm(A: torch.Tensor, vals: torch.Tensor, meta: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    D = torch.empty((A.shape[0], vals.shape[0]), dtype=torch.bfloat16, device=A.device)
+    api.sparse24_gemm(_bytes(A), vals, meta, D, scale, check=True)
+    return D
+
+
+@sparse24_gemm.register_fake
+def _(A, vals, meta, scale):
+    return A.new_empty((A.shape[0], vals.shape[0]), dtype=torch.bfloat16)

@@ -1,0 +1,86 @@
+"""The registered torch operators (torch.ops.sgemm.*): schemas and shape inference on the CPU, results and
+torch.compile tracing on the GPU.  The reference's counterpart is its pybind extension
+(skinny_gemm/skinny_gemm_binding.cu:64-100), mirrored by rocm_dev_amd.HFRK_skinny_gemm; these are the functional
+operators torch.library and torch.compile see."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import GEMM_TOL, bits, dev, gemm_reference, scale_tensor
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import rocm_dev_amd.torch_ops  # noqa: F401  (registers the operators)
+    return torch.ops.sgemm
+
+
+def test_operators_are_registered_with_schemas(ops):
+    for name in ("skinny_gemm", "skinny_gemm_rowcol", "skinny_gemm_bf16act", "fp8_encode_rows", "fp8_decode_rows", "sparse24_gemm"):
+        op = getattr(ops, name).default
+        assert "sgemm::" + name in str(op._schema)
+    assert "Tensor? row_scales=None" in str(ops.skinny_gemm_rowcol.default._schema)
+
+
+def test_shape_inference_on_meta_tensors(ops):
+    A = torch.empty((8, 512), dtype=torch.uint8, device="meta")
+    W = torch.empty((96, 512), dtype=torch.uint8, device="meta")
+    s = torch.empty((1,), dtype=torch.float32, device="meta")
+    X = torch.empty((8, 512), dtype=torch.bfloat16, device="meta")
+    assert ops.skinny_gemm(A, W, s).shape == (8, 96) and ops.skinny_gemm(A, W, s).dtype == torch.bfloat16
+    assert ops.skinny_gemm_rowcol(A, W).shape == (8, 96)
+    assert ops.skinny_gemm_bf16act(X, W, s).shape == (8, 96)
+    q, r = ops.fp8_encode_rows(X)
+    assert q.shape == (8, 512) and q.dtype == torch.uint8 and r.shape == (8,) and r.dtype == torch.float32
+    assert ops.fp8_decode_rows(q, r).dtype == torch.bfloat16
+    vals = torch.empty((96, 256), dtype=torch.uint8, device="meta")
+    meta = torch.empty((96, 64), dtype=torch.uint8, device="meta")
+    assert ops.sparse24_gemm(A, vals, meta, s).shape == (8, 96)
+
+
+@pytest.mark.gpu
+def test_results_equal_the_c_abi(ops, oracle):
+    import rocm_dev_amd as sg
+    m, n, k = 8, 1024, 4096
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=2)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    D = ops.skinny_gemm(A, B, S)
+    want = torch.empty_like(D)
+    assert sg.skinny_gemm_fastpath(A, B, want, S) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(D, want)
+    assert oracle.max_rel_err_bf16(bits(D), gemm_reference(oracle, a8, b8, scale)) <= GEMM_TOL
+    # float8 tensors are taken as they are
+    assert torch.equal(ops.skinny_gemm(A.view(torch.float8_e4m3fn), B.view(torch.float8_e4m3fn), S), want)
+    # encode -> rowcol == bf16act, and decode(encode(x)) equals the oracle's
+    x = oracle.normal_bf16_outliers((m, k), seed=4, stream_id=3)
+    X = dev(x)
+    q, r = ops.fp8_encode_rows(X)
+    q_ref, s_ref = oracle.fp8_encode_rows(x)
+    assert np.array_equal(q.cpu().numpy(), q_ref) and np.array_equal(r.cpu().numpy(), s_ref)
+    assert np.array_equal(bits(ops.fp8_decode_rows(q, r)), oracle.fp8_decode_rows(q_ref, s_ref))
+    two = ops.skinny_gemm_rowcol(q, B, S, r, None)
+    one = ops.skinny_gemm_bf16act(X, B, S, None)
+    assert torch.equal(one, two)
+    a8s, vals, meta, _, sc = oracle.make_sparse24_operands(m, 512, 2048, seed=3)
+    Ds = ops.sparse24_gemm(dev(a8s), dev(vals), dev(meta), scale_tensor(sc))
+    assert oracle.max_rel_err_bf16(bits(Ds), oracle.gemm_sparse24(a8s, vals, meta, sc)) <= GEMM_TOL
+
+
+@pytest.mark.gpu
+def test_opcheck_and_compile(ops, oracle):
+    m, n, k = 8, 512, 1024
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=5)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    torch.library.opcheck(ops.skinny_gemm.default, (A, B, S), test_utils=("test_schema", "test_faketensor"))
+    X = dev(oracle.normal_bf16_outliers((m, k), seed=6, stream_id=3))
+    torch.library.opcheck(ops.fp8_encode_rows.default, (X,), test_utils=("test_schema", "test_faketensor"))
+
+    def layer(x, w, s):
+        q, r = torch.ops.sgemm.fp8_encode_rows(x)
+        return torch.ops.sgemm.skinny_gemm_rowcol(q, w, s, r, None).float() * 2.0
+
+    eager = layer(X, B, S)
+    compiled = torch.compile(layer, backend="aot_eager", fullgraph=True)(X, B, S)
+    torch.cuda.synchronize()
+    assert torch.equal(eager, compiled)
