@@ -52,6 +52,7 @@ def main():
                     help="fill the operands with uniformly random E4M3 codes from torch's generator (one kernel per buffer) "
                          "instead of the seeded N(0,1) recipe (dozens of elementwise kernels per buffer): for profiler runs "
                          "that serialise every dispatch; timings of such a run are not the benchmark's")
+    ap.add_argument("--tuning", help="tuning table to load first (sg_tuning_load): every mode then runs the table's records")
     ap.add_argument("--replays", type=int, default=31, help="timed regions per measurement (the median is reported)")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
@@ -103,6 +104,8 @@ def main():
     torch.manual_seed(0)
     if lib.sg_init() != 0:
         sys.exit("bench.py: sg_init failed")
+    if args.tuning and lib.sg_tuning_load(args.tuning.encode()) != 0:
+        sys.exit("bench.py: cannot load tuning table %s" % args.tuning)
 
     if args.n_sweep:
         import ctypes

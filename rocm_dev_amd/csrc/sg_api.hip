@@ -585,6 +585,8 @@ static int check_pointers(const void* A, const void* B, const void* D, int m, in
     if (!A || !B || !D || m <= 0 || n <= 0 || k <= 0 || b_stride < k) return SG_BAD_ARGUMENT;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15u) return SG_BAD_ALIGNMENT;
     if ((reinterpret_cast<uintptr_t>(D) & 7u) || (b_stride & 15)) return SG_BAD_ALIGNMENT;
+    // the kernels address a tile's rows with 32-bit offsets from the tile's first row: 64 rows must stay below 2 GB
+    if ((size_t)b_stride * 64 > 0x7fffffffu || (size_t)k * 64 > 0x7fffffffu) return SG_BAD_ARGUMENT;
     return SG_SUCCESS;
 }
 
@@ -682,9 +684,11 @@ static Config pick_config(int m, int n, int k, int cu_count) {
                 c.depth = 3;
             }
         } else {                                // about one tile per CU: few waves, deep rings
+            // (one wave x eight slots also for long K: 4096 x 14336 at 1, 4, 8, 16 rows 0.5-2.3 % ahead of two waves
+            // x four slots in the tuner's alternating rounds - no cross-wave reduction in front of the store)
             c.rg = 1;
-            c.waves = blocks >= 48 ? 2 : 1;
-            c.depth = c.waves == 1 ? 8 : 4;
+            c.waves = 1;
+            c.depth = 8;
             // between one and two 16-row tiles per CU half of the CUs stream twice what the others do (all
             // workgroups are resident at once); 24-row tiles that give every CU one workgroup level that.  Measured
             // on 6144 x 4096: level with 16-row tiles up to 8 activation rows (6.75 against 6.70 us - the launch is

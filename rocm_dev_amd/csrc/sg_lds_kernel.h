@@ -413,7 +413,7 @@ lds_gemm_persistent_kernel(const StreamArgs a) {
     // a store in their vmcnt queue (a store younger than the ring's DMAs makes every later
     // vmcnt(n) wait for one DMA more than needed until the store is acknowledged)
     const bool epilogue_wave = blockDim.x > (unsigned)waves * 64;
-    const int per_tile = (wave < waves && wave < blocks) ? (blocks - wave + waves - 1) / waves : 0;
+    const int per_tile = wave < waves ? blocks_of_wave(a, blocks, wave) : 0;
     const int total = per_tile * my_tiles;
 
     const int q = lane >> 2, p = lane & 3;
@@ -429,35 +429,55 @@ lds_gemm_persistent_kernel(const StreamArgs a) {
     float* xscale = reinterpret_cast<float*>(red + (size_t)2 * FRAGS * waves * 64);
     const float* row_factors = quant ? xscale : nullptr;
 
-    auto tile_origin = [&](int j, int& m0, int& n0) __attribute__((always_inline)) {  // j-th tile of this workgroup
-        const int t = run.first + j;
-        n0 = (t % a.n_tiles) * (16 * RG);
-        m0 = (t / a.n_tiles) * (16 * MT);
-    };
+    // Tiles are walked n fastest.  Both the issuing and the finishing side keep their tile's (n, m) coordinates as
+    // counters that are stepped when a tile ends: dividing by run-time values per stage (tile index, tile
+    // coordinates) cost about 0.8 us in front of the first DMA and delayed every refill.
+    const unsigned first_m = fast_div((unsigned)run.first, (unsigned)a.n_tiles, a.inv_n_tiles);
+    const int first_n = run.first - (int)first_m * a.n_tiles;
+    int iss_tn = first_n, iss_tm = (int)first_m, iss_r = 0;     // tile and stage-in-tile of the next stage to issue
+    int fin_tn = first_n, fin_tm = (int)first_m;                // tile the next tile_done() finishes
 
-    auto issue = [&](int i) __attribute__((always_inline)) {
-        const int j = i / per_tile;
-        const int kb = wave + (i - j * per_tile) * waves;
-        int m0, n0;
-        tile_origin(j, m0, n0);
+    // per-lane parts of the DMA addresses: row inside the tile and byte offset inside the 256-byte K block; the rest
+    // of an address (tile origin, K block) is wave-uniform and travels in scalar registers
+    int wrow[RG][4];
+    unsigned wcol[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        wcol[u] = src_col + ((p + u) & 3) * 16;
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) wrow[rg][u] = rg * 16 + 4 * u + src_row;
+    }
+
+    auto issue = [&](int i) __attribute__((always_inline)) {   // called for i = 0, 1, 2, ... in order
+        const int kb = wave + iss_r * waves;
+        const int n0 = iss_tn * (16 * RG), m0 = iss_tm * (16 * MT);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
-        const size_t koff = ((size_t)kb << 8) + src_col;
+        const uint8_t* w_base = a.B + (size_t)n0 * a.b_stride + ((size_t)kb << 8);
+        const int w_last = a.n - 1 - n0;     // rows past the edge re-read the last row, never stored
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                int row = n0 + rg * 16 + 4 * u + src_row;
-                row = row < a.n ? row : a.n - 1;
-                const uint8_t* src = a.B + (size_t)row * a.b_stride + koff + ((p + u) & 3) * 16;
-                if (NT) dma_1kb_stream(src, slot + (rg * 4 + u) * 1024);
-                else dma_1kb(src, slot + (rg * 4 + u) * 1024);
+                const int row = wrow[rg][u] < w_last ? wrow[rg][u] : w_last;
+                const unsigned voff = (unsigned)row * (unsigned)a.b_stride + wcol[u];
+                if (NT) dma_1kb_stream_at(w_base, voff, slot + (rg * 4 + u) * 1024);
+                else dma_1kb_at(w_base, voff, slot + (rg * 4 + u) * 1024);
             }
         if (!XRES) {
+            const uint8_t* x_base = a.A + (size_t)m0 * a.k + ((size_t)kb << 8);
+            const int x_last = a.m - 1 - m0;
 #pragma unroll
             for (int u = 0; u < XU; u++) {
-                int row = m0 + 4 * u + src_row;
-                row = row < a.m ? row : a.m - 1;
-                dma_1kb(a.A + (size_t)row * a.k + koff + ((p + (u & 3)) & 3) * 16, slot + (RG * 4 + u) * 1024);
+                int row = 4 * u + src_row;
+                row = row < x_last ? row : x_last;
+                dma_1kb_at(x_base, (unsigned)row * (unsigned)a.k + wcol[u & 3], slot + (RG * 4 + u) * 1024);
+            }
+        }
+        if (++iss_r == per_tile) {
+            iss_r = 0;
+            if (++iss_tn == a.n_tiles) {
+                iss_tn = 0;
+                iss_tm++;
             }
         }
     };
@@ -478,10 +498,14 @@ lds_gemm_persistent_kernel(const StreamArgs a) {
     };
 
     const float scale = a.scale ? a.scale[0] : 1.0f;
+    int red_turn = 0;
     // Reduce the waves' partial tiles of the j-th tile in wave order, scale, round, store.
     auto tile_done = [&](int j) __attribute__((always_inline)) {
-        int m0, n0;
-        tile_origin(j, m0, n0);
+        const int n0 = fin_tn * (16 * RG), m0 = fin_tm * (16 * MT);
+        if (++fin_tn == a.n_tiles) {
+            fin_tn = 0;
+            fin_tm++;
+        }
         if (waves == 1 && !epilogue_wave) {
 #pragma unroll
             for (int f = 0; f < FRAGS; f++)
@@ -500,8 +524,9 @@ lds_gemm_persistent_kernel(const StreamArgs a) {
             __syncthreads();
             // without an epilogue wave the reducing wave rotates with the tile, so that the cost is
             // spread over the waves
-            int first = wave - j % waves, step = waves;
+            int first = wave - red_turn, step = waves;        // red_turn = j % waves, kept as a counter
             first = first < 0 ? first + waves : first;
+            red_turn = red_turn + 1 == waves ? 0 : red_turn + 1;
             if (epilogue_wave) {
                 first = wave == waves ? 0 : FRAGS;
                 step = 1;
