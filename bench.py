@@ -147,7 +147,7 @@ def main():
             fns = (lambda i, st: lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, st),
                    lambda i, st: lib.sg_skinny_gemm_tuned(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k,
                                                           ctypes.byref(per_tile), st),
-                   lambda i, st: lib.sg_debug_read_stream(wb[i % copies].data_ptr(), n, k, k, st))
+                   lambda i, st: lib.sg_debug_read_stream(wb[i % copies].data_ptr(), n, k, k, 256, st))
             t = [graph_us(f) for f in fns]
             mb = gemm_bytes(m, n, k) / 1e6
             print("| %d | %.1f | %.1f | %.2f | %.2f | %.2f |" % (n, n / 16 / 256, mb, t[0], t[1], t[2]), flush=True)
@@ -198,7 +198,7 @@ def main():
         n, k = SHAPES["gate_up"]
         wb = [synth.quantize_tensor(synth.normal_f32((n, k), c, 2))[0] for c in range(6)]
         for i in range(6):
-            lib.sg_debug_read_stream(wb[i].data_ptr(), n, k, k, None)
+            lib.sg_debug_read_stream(wb[i].data_ptr(), n, k, k, 256, None)
         torch.cuda.synchronize()
         return
 

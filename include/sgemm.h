@@ -226,11 +226,13 @@ int sg_tuning_save(const char* path);
  * no other thread launches.  sg_debug_stamps(NULL, 0) switches the stamps off again. */
 int sg_debug_stamps(unsigned long long* device_buffer, size_t n_words);
 
-/* Profiling aid, no counterpart in the reference: reads the n x k weight matrix B (row stride b_stride, k % 256 == 0)
- * exactly the way the persistent LDS-ring GEMM streams it - one workgroup per CU walking 16-row tiles, eight waves
- * sharing K, 4 rows x 256 B direct-to-LDS loads with the streaming hint - and does nothing with it.  Its duration
- * is the ceiling of that access pattern on the device: what a GEMM's streaming phase is measured against. */
-int sg_debug_read_stream(const uint8_t* B, int n, int k, int b_stride, void* stream);
+/* Profiling aid, no counterpart in the reference: reads the n x k weight matrix B (row stride b_stride, k % 1024 == 0)
+ * the way the persistent LDS-ring GEMM streams it - one workgroup per CU walking row tiles, eight waves sharing K,
+ * direct-to-LDS loads with the streaming hint, two 4 KB slots per wave - and does nothing with it.  Its duration is the
+ * ceiling of that access pattern on the device: what a GEMM's streaming phase is measured against.  segment_bytes is
+ * what one load instruction takes contiguously from one row: 256 (4 rows per instruction - the GEMM's own pattern),
+ * 512 (2 rows) or 1024 (1 row). */
+int sg_debug_read_stream(const uint8_t* B, int n, int k, int b_stride, int segment_bytes, void* stream);
 
 /* Replaces  template<class out> void async_gemm(const fp8* A, const fp8* B, out* D, int m,
  * int n, int k)  (async_gemm_sparse/sparse_k.cu:45-69, async_gemm_blanes/sparse_k.cu,

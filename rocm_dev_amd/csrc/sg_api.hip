@@ -898,14 +898,17 @@ int sg_debug_stamps(unsigned long long* device_buffer, size_t n_words) {
     return SG_SUCCESS;
 }
 
-int sg_debug_read_stream(const uint8_t* B, int n, int k, int b_stride, void* stream) {
-    if (!B || n <= 0 || k <= 0 || k % 256 != 0 || b_stride < k || (b_stride & 15) || (reinterpret_cast<uintptr_t>(B) & 15u))
+int sg_debug_read_stream(const uint8_t* B, int n, int k, int b_stride, int segment_bytes, void* stream) {
+    if (!B || n <= 0 || k <= 0 || k % 1024 != 0 || b_stride < k || (b_stride & 15) || (reinterpret_cast<uintptr_t>(B) & 15u))
         return SG_BAD_ARGUMENT;
+    if (segment_bytes != 256 && segment_bytes != 512 && segment_bytes != 1024) return SG_BAD_ARGUMENT;
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
-    const int tiles = (n + 15) / 16;
+    const int tile_rows = 4 * (1024 / segment_bytes);
+    const int tiles = (n + tile_rows - 1) / tile_rows;
     const unsigned grid = (unsigned)(tiles < dev->cu_count ? tiles : dev->cu_count);
-    read_stream_kernel<<<dim3(grid), dim3(512), 8 * 2 * 4096, static_cast<hipStream_t>(stream)>>>(B, n, k, b_stride, nullptr);
+    auto kernel = segment_bytes == 256 ? read_stream_kernel<256> : (segment_bytes == 512 ? read_stream_kernel<512> : read_stream_kernel<1024>);
+    kernel<<<dim3(grid), dim3(512), 8 * 2 * 4096, static_cast<hipStream_t>(stream)>>>(B, n, k, b_stride, nullptr);
     return report_hip("read_stream_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }
 

@@ -8,28 +8,31 @@
 
 namespace sg {
 
+// SEG: contiguous bytes a DMA instruction takes from one row - 256 (4 rows per instruction, the GEMM's pattern), 512
+// (2 rows) or 1024 (1 row); a wave's stage is always 4 KB = 4 instructions: 16 rows x 256 B, 8 x 512 B or 4 x 1 KB.
+template <int SEG>
 __global__ void __launch_bounds__(512) read_stream_kernel(const uint8_t* B, int n, int k, int b_stride, unsigned* sink) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];   // [wave][2][4 KB]
     constexpr int DEPTH = 2, PER_STAGE = 4, STAGE_BYTES = 4096;
     const int lane = lane_id(), wave = wave_id(), waves = (int)blockDim.x >> 6;
-    const int blocks = k >> 8;
-    const TileRun run = persistent_tile_run((n + 15) / 16);
+    constexpr int ROWS_PER_INSTR = 1024 / SEG, TILE_ROWS = 4 * ROWS_PER_INSTR;   // 16, 8 or 4 rows per tile
+    const int blocks = k / SEG;
+    const TileRun run = persistent_tile_run((n + TILE_ROWS - 1) / TILE_ROWS);
     const int per_tile = wave < blocks ? (blocks - wave + waves - 1) / waves : 0;
     const int total = per_tile * run.count;
-    const int q = lane >> 2, p = lane & 3;
-    const int src_row = q & 3, src_col = (q >> 2) * 64;
+    const int src_row = (lane * 16) / SEG, src_col = (lane * 16) % SEG;   // 16 bytes per lane, lanes in address order
     const unsigned my_ring_lds = lds_addr(ring + (size_t)wave * (DEPTH * STAGE_BYTES));
     const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
     auto issue = [&](int i) __attribute__((always_inline)) {
         const int j = i / per_tile;
         const int kb = wave + (i - j * per_tile) * waves;
-        const int n0 = (run.first + j) * 16;
+        const int n0 = (run.first + j) * TILE_ROWS;
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            int row = n0 + 4 * u + src_row;
+            int row = n0 + ROWS_PER_INSTR * u + src_row;
             row = row < n ? row : n - 1;
-            dma_1kb_stream(B + (size_t)row * b_stride + ((size_t)kb << 8) + src_col + ((p + u) & 3) * 16, slot + u * 1024);
+            dma_1kb_stream(B + (size_t)row * b_stride + (size_t)kb * SEG + src_col, slot + u * 1024);
         }
     };
     unsigned seen = 0;
