@@ -666,9 +666,12 @@ def main():
         tbb = torch.randn((tb, tm, tn), device="cuda", dtype=torch.float32)
         td = torch.empty((tm, tn), device="cuda", dtype=torch.float32)
         tsr_us = graph_time_us(lambda i, st: lib.sg_tiled_sum_reduce(ta.data_ptr(), tbb.data_ptr(), td.data_ptr(), tb, tm, tn, st), 8)
+        tsr_q_us = graph_time_us(lambda i, st: lib.sg_tiled_sum_reduce_async(ta.data_ptr(), tbb.data_ptr(), td.data_ptr(), tb, tm, tn, st), 8)
         tsr_bytes = (2 * tb + 1) * tm * tn * 4
         others["tiled_sum_reduce_8x1024x8192"] = {"us": round(tsr_us, 2), "TBps": round(tsr_bytes / tsr_us / 1e6, 3),
-                                                  "note": "reads 512 MiB per launch (beyond the 256 MB cache), writes 32 MiB"}
+                                                  "lds_queue_us": round(tsr_q_us, 2), "lds_queue_TBps": round(tsr_bytes / tsr_q_us / 1e6, 3),
+                                                  "note": "reads 512 MiB per launch (beyond the 256 MB cache), writes 32 MiB; "
+                                                          "lds_queue = sg_tiled_sum_reduce_async"}
         del ta, tbb, td
         # bf16 activations quantised per row inside the GEMM (one launch) against the two launches it replaces
         # (sg_fp8_encode_rows, then sg_skinny_gemm_rowcol with the library's own configuration), cold weights

@@ -273,6 +273,13 @@ int sg_sparse24_compress(const uint8_t* B, uint8_t* B_vals, uint8_t* B_meta, int
  * in batch order per element.  Any m, n (the reference needs m % 8 == 0, n % 64 == 0). */
 int sg_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n, void* stream);
 
+/* Replaces  void tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n)  of
+ * tiled_sum_reduce_async/src.cu:179-200, the variant that stages the batches through a queue in LDS
+ * (kernel :98-177, producers :13-48, consumers :50-96).  Same result bits as sg_tiled_sum_reduce; every
+ * wave keeps its own queue of direct-to-LDS loads, two to four batches ahead, ordered by its load counter
+ * instead of flag bytes.  Any b, m, n. */
+int sg_tiled_sum_reduce_async(const float* A, const float* B, float* D, int b, int m, int n, void* stream);
+
 /* Per-row FP8 codec - no counterpart in the reference; the local compute on either side
  * of an FP8 all-reduce exchange.
  *   encode: scales[r] = absmax(X[r,:]) / 448 (1 if the row is all zero; NaNs do not count towards the maximum),

@@ -40,9 +40,14 @@ inline int async_gemm<unsigned short>(const fp8* A, const fp8* B, unsigned short
     return sg_async_gemm_bf16(A, B, D_bf16, m, n, k);
 }
 
-/* tiled_sum_reduce/src.cu:52-59 */
+/* tiled_sum_reduce/src.cu:52-59; define SGEMM_COMPAT_TSR_ASYNC before including this header to get the launcher of
+ * tiled_sum_reduce_async/src.cu:179-200 (same name, same arguments, batches staged through a queue in LDS) instead */
 inline int tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n) {
+#ifdef SGEMM_COMPAT_TSR_ASYNC
+    return sg_tiled_sum_reduce_async(A, B, D, b, m, n, nullptr);
+#else
     return sg_tiled_sum_reduce(A, B, D, b, m, n, nullptr);
+#endif
 }
 
 #endif /* SGEMM_COMPAT_HPP */

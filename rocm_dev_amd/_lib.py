@@ -46,6 +46,7 @@ SIGNATURES = {
     "sg_sparse24_gemm_tuned": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "sg_sparse24_compress": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sg_tiled_sum_reduce": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sg_tiled_sum_reduce_async": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sg_fp8_encode_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "sg_fp8_decode_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "sg_fp8_reduce_rows": (_i, [_vp, _vp, _vp, _i, _sz, _i, _i, _vp]),

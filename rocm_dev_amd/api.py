@@ -5,7 +5,7 @@ Reference interfaces mirrored (paths below the reference's projects/ directory):
   skinny_gemm_fastpath(...)   skinny_gemm/skinny_gemm_caller.cu:343-346
   HFRK_skinny_gemm            skinny_gemm/skinny_gemm_binding.cu:64-100
   async_gemm(...)             async_gemm_sparse/sparse_k.cu:45-69
-  tiled_sum_reduce(...)       tiled_sum_reduce/src.cu:52-73
+  tiled_sum_reduce(...)       tiled_sum_reduce/src.cu:52-73, tiled_sum_reduce_async/src.cu:179-200 (lds_queue=True)
 Every function returns the integer return code of the C ABI (0 = success), as the
 reference's launchers do; ``check=True`` raises SgError instead.  Tensors are torch CUDA
 tensors used purely as device buffers: fp8 operands are uint8 or float8_e4m3fn, outputs
@@ -302,12 +302,13 @@ def async_gemm(A, B, D, check=False):
     return _done(rc, check)
 
 
-def tiled_sum_reduce(A, B, D, check=False):
-    """D[m,n] = sum_b (A[b,m,n] + B[b,m,n]) in fp32, batch order."""
+def tiled_sum_reduce(A, B, D, check=False, lds_queue=False):
+    """D[m,n] = sum_b (A[b,m,n] + B[b,m,n]) in fp32, batch order.  lds_queue=True runs the variant that stages the
+    batches through a queue in LDS (tiled_sum_reduce_async/src.cu:179-200); the result bits are the same."""
     b, m, n = A.shape
+    fn = lib.sg_tiled_sum_reduce_async if lds_queue else lib.sg_tiled_sum_reduce
     with torch.cuda.device(A.device):
-        rc = lib.sg_tiled_sum_reduce(_dev(A, torch.float32), _dev(B, torch.float32), _dev(D, torch.float32),
-                                     b, m, n, _stream())
+        rc = fn(_dev(A, torch.float32), _dev(B, torch.float32), _dev(D, torch.float32), b, m, n, _stream())
     return _done(rc, check)
 
 

@@ -22,6 +22,7 @@ int launch_fp8_decode_rows(const uint8_t* Q, const float* scales, void* Y, int r
 int launch_fp8_reduce_rows(const uint8_t* Q, const float* scales, void* Y, int nbuf, size_t q_buf_stride, int rows,
                            int cols, hipStream_t stream);
 int launch_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n, hipStream_t stream);
+int launch_tiled_sum_reduce_ring(const float* A, const float* B, float* D, int b, int m, int n, hipStream_t stream);
 int launch_sparse24_compress(const uint8_t* B, uint8_t* vals, uint8_t* meta, int n, int k, int b_stride, hipStream_t stream);
 
 // ---- per-device state -------------------------------------------------------------------
@@ -1355,6 +1356,10 @@ int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_
 
 int sg_tiled_sum_reduce(const float* A, const float* B, float* D, int b, int m, int n, void* stream) {
     return launch_tiled_sum_reduce(A, B, D, b, m, n, static_cast<hipStream_t>(stream));
+}
+
+int sg_tiled_sum_reduce_async(const float* A, const float* B, float* D, int b, int m, int n, void* stream) {
+    return launch_tiled_sum_reduce_ring(A, B, D, b, m, n, static_cast<hipStream_t>(stream));
 }
 
 int sg_fp8_encode_rows(const void* X, uint8_t* Q, float* scales, int rows, int cols, void* stream) {
