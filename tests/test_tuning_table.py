@@ -172,3 +172,39 @@ def test_heuristics_pick_the_fourteen_wave_tile_where_it_fills_the_chip():
     for m, n in ((64, 57344 + 128), (300, 57344)):
         t, _ = api.skinny_gemm_choice(m, n, 8192)
         assert t.waves != 14, (m, n)
+
+
+def test_the_heuristics_only_choose_what_the_launchers_take():
+    """A sweep of shapes through the library's own choice (no table): whatever engine it names, the record must be one
+    the launch rules - written down independently of the launchers - accept, so a legal shape cannot fail in the
+    fastpath because the heuristics picked a configuration that does not fit.  (The launchers fall back when a choice is
+    refused; this is the check that they never need to.)"""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(__file__))
+    import launch_rules
+    import rocm_dev_amd as sg
+    sg.tuning_clear()
+    ms = [1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 256, 300, 512]
+    ns = [2, 16, 18, 256, 1000, 4096, 4112, 6144, 8192, 10240, 14336, 28672, 57344, 128256]
+    ks = [256, 512, 768, 1024, 2048, 4096, 5120, 8192, 14336, 28672]
+    checked = {1: 0, 2: 0, 4: 0}
+    for m in ms:
+        for n in ns:
+            for k in ks:
+                choice, from_table = sg.skinny_gemm_choice(m, n, k)
+                assert not from_table
+                r = autotune_fields(choice)
+                checked[r["engine"]] += 1
+                if r["engine"] == autotune.ENGINE_LDS:
+                    assert m <= 32 and launch_rules.expect_lds(m, n, k, r) == launch_rules.OK, (m, n, k, r)
+                elif r["engine"] == autotune.ENGINE_MID:
+                    assert launch_rules.expect_mid(m, n, k, r) == launch_rules.OK, (m, n, k, r)
+                else:
+                    assert r["engine"] == autotune.ENGINE_DIRECT and r["m_blocks"] in (1, 2), (m, n, k, r)
+    assert checked[2] > 1000 and checked[4] > 1000, checked
+    # k the LDS engines cannot take goes to the direct engine, for every m
+    for m in (1, 8, 32, 64):
+        for k in (16, 48, 4096 + 64):
+            choice, _ = sg.skinny_gemm_choice(m, 4096, k)
+            assert choice.engine == autotune.ENGINE_DIRECT, (m, k)
