@@ -254,6 +254,16 @@ static int launch_stream(const Config& c, StreamArgs a, hipStream_t stream) {
     return SG_INVALID_CONFIG;
 }
 
+// Persistent workgroups for `tiles` tiles when at most `most` fit the device: the launch lasts as long as the
+// workgroup with the most tiles, ceil(tiles / most) of them, so no more workgroups are started than it takes to give
+// every one that many (896 tiles on 256 CUs: 224 workgroups of 4 instead of 128 of 4 and 128 of 3 - the same
+// critical path with fewer streams competing for memory, 8 x 14336 x 4096 12.35 -> 11.54 us).
+static unsigned level_persistent_grid(unsigned tiles, size_t most) {
+    if (most >= tiles) return tiles;
+    const size_t rounds = (tiles + most - 1) / most;
+    return (unsigned)((tiles + rounds - 1) / rounds);
+}
+
 static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     if (a.k % 256 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     // wave_tiles bit 3: 24-row tiles (two fragments, the second half used), one workgroup per tile
@@ -292,8 +302,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         if (pt * c.mt > 4) return SG_INVALID_CONFIG;
         DeviceInfo* dev;
         if (int rc = get_device_info(&dev)) return rc;
-        const size_t want = (size_t)dev->cu_count * c.persist;
-        if (want < grid) grid = (unsigned)want;
+        grid = level_persistent_grid(grid, (size_t)dev->cu_count * c.persist);
         const unsigned threads = (unsigned)(c.waves + ((c.wavetile & 4) ? 1 : 0)) * 64;
         if (threads > 1024) return SG_TOO_MANY_WARPS;
         const size_t lds_x = (size_t)c.waves * c.depth * c.rg * 4096 + 2u * c.waves * c.rg * c.mt * 1024;
@@ -311,8 +320,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         lds += 2u * c.waves * c.rg * c.mt * 1024;   // double-buffered reduction scratch
         DeviceInfo* dev;
         if (int rc = get_device_info(&dev)) return rc;
-        const size_t want = (size_t)dev->cu_count * c.persist;
-        if (want < grid) grid = (unsigned)want;
+        grid = level_persistent_grid(grid, (size_t)dev->cu_count * c.persist);
     }
     if (lds > 159 * 1024) return SG_INVALID_CONFIG;  // 160 KB per CU, minus the kernel's static LDS
     if (a.A16) {   // only the resident-activation kernel quantises bf16 activations itself
