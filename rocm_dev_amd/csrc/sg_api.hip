@@ -436,7 +436,7 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
 // possible, then the tile: 128x128 and 128x64 tiles on eight waves beat both smaller tiles
 // (more operand traffic per flop) and 256-wide ones (one workgroup per CU and a two-slot ring),
 // which only pay off when nothing else fits in one round.  K may be split up to four ways as
-// long as every split keeps 32 K blocks.
+// long as every split keeps 32 K blocks (three ways: 16, for m <= 64).
 static Config pick_mid(int m, int n, int k, int cu_count) {
     struct Tile { int bn, bm, waves; };
     // {224, *, 14}: fourteen waves; 57344 = 256 x 224 gives every CU a tile where 256-row tiles fill 224 of 256
@@ -450,8 +450,10 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     for (const Tile& t : order) {
         if (t.bm > bm_max) continue;
         const long tiles = (long)((n + t.bn - 1) / t.bn) * ((m + t.bm - 1) / t.bm);
-        for (int sk = 1; sk <= 4; sk *= 2) {
-            if (sk > 1 && blocks / sk < 32) break;
+        for (int sk = 1; sk <= 4; sk++) {
+            // a three-way split only up to 64 activation rows, where the partials are small against the weights
+            // (64 x 10240 x 8192: 80 tiles -> 240 workgroups, 24.5 -> 22.5 us); two and four ways keep 32 K blocks
+            if (sk == 3 ? (m > 64 || blocks / sk < 16) : (sk > 1 && blocks / sk < 32)) continue;
             const long wgs = tiles * sk;
             const long rounds = (wgs + cu_count - 1) / cu_count;
             // the fourteen-wave tile only where it is known to pay: unsplit, one tile covering all of m (the
