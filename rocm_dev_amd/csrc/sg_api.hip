@@ -305,8 +305,13 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         grid = level_persistent_grid(grid, (size_t)dev->cu_count * c.persist);
         const unsigned threads = (unsigned)(c.waves + ((c.wavetile & 4) ? 1 : 0)) * 64;
         if (threads > 1024) return SG_TOO_MANY_WARPS;
-        const size_t lds_x = (size_t)c.waves * c.depth * c.rg * 4096 + 2u * c.waves * c.rg * c.mt * 1024;
+        size_t lds_x = (size_t)c.waves * c.depth * c.rg * 4096 + 2u * c.waves * c.rg * c.mt * 1024;
         if (lds_x > 159 * 1024) return SG_INVALID_CONFIG;
+        // room for one more 4 KB staging block per wave (the kernel has no static LDS: all 160 KB may be asked for):
+        // the activation fragments then reach the registers without the first weight stages being waited for
+        a.x_extra = (c.mt == 2 && pt == 2 && lds_x + (size_t)c.waves * 4096 <= 160 * 1024) ? 1 : 0;
+        if (a.x_extra) lds_x += (size_t)c.waves * 4096;
+        a.stamps = take_stamps(grid);
         return launch_xreg(c.mt, c.rg, pt, c.depth, a, grid, threads, lds_x, stream);
     } else if (c.persist > 0) {
         if (c.split_k != 1) return SG_INVALID_CONFIG;

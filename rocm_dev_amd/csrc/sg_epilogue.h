@@ -35,6 +35,7 @@ struct StreamArgs {
     int out_f32;
     unsigned inv_n_tiles, inv_split_k, inv_waves;  // div_reciprocal() of n_tiles, split_k, waves (set_reciprocals)
     unsigned long long* stamps;  // profiling aid, normally nullptr: kStampWords time stamps per workgroup (sg_debug_stamps)
+    int x_extra;            // register-resident kernel: 1 = the launch's LDS has one more 4 KB staging block per wave behind the reduction scratch
 };
 
 // Time stamps a workgroup leaves when a.stamps is set (wave 0 writes them when it is done):

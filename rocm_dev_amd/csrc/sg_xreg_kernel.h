@@ -3,9 +3,9 @@
 // In the persistent K-split kernel (sg_lds_kernel.h) wave w of a workgroup always works on K
 // blocks w, w + waves, ... of whatever tile the workgroup is at.  When the K range is short enough
 // that this is PT <= 4 blocks per wave, the activation fragments of exactly those blocks - the
-// same for every tile - fit in the wave's registers (16*PT*MT VGPRs): they are loaded once, in
-// MFMA operand layout, straight from global memory, and for the rest of the kernel the ring
-// carries weights only and no activation byte crosses L2 or LDS again.  That removes what makes
+// same for every tile - fit in the wave's registers (16*PT*MT VGPRs): they are loaded once
+// (through LDS, in the weights' own load pattern, see the prologue), and for the rest of the kernel
+// the ring carries weights only and no activation byte crosses L2 or LDS again.  That removes what makes
 // M = 17..32 slow in the other variants (an 8 KB activation stage next to every 16 KB weight
 // stage) and frees the LDS the resident-in-LDS variant spends on the activations.
 //
@@ -34,11 +34,13 @@ template <int MT, int RG, int PT, int DEPTH, bool NT>
 __global__ void __launch_bounds__(xreg_launch_bound(MT, RG, PT)) lds_gemm_xreg_kernel(const StreamArgs a) {
     // [wave][DEPTH][RG*4 KB] | red[2][FRAGS][wave][64] f32x4
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
+    Stamps stamps;
+    stamps.begin();
 
     constexpr int PER_STAGE = RG * 4;
     constexpr int STAGE_BYTES = PER_STAGE * 1024;
     constexpr int FRAGS = RG * MT;
-    static_assert((DEPTH - 1) * PER_STAGE <= 63, "ring deeper than vmcnt can count");
+    static_assert((DEPTH - 1) * PER_STAGE + 4 <= 63, "ring deeper than vmcnt can count");
     static_assert(PT * MT <= 4, "activation fragments must fit in registers");
 
     const int lane = lane_id();
@@ -142,42 +144,114 @@ __global__ void __launch_bounds__(xreg_launch_bound(MT, RG, PT)) lds_gemm_xreg_k
             for (int mt = 0; mt < MT; mt++) acc[rg][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     };
 
-    if (!streaming) {   // epilogue wave: takes part in every tile's barrier, reduces and stores
+    if (!streaming) {   // epilogue wave: takes part in every barrier, reduces and stores
+        __syncthreads();   // the reduction scratch is free (it staged activations, see below)
         for (int j = 0; j < my_tiles; j++) tile_done(j);
         return;
     }
 
-    for (int d = 0; d < DEPTH && d < total; d++) issue(d);
-
-    // ---- activations: once, into registers ------------------------------------------------------
-    // Loaded after the first stages have been issued, and waited for with the builtin (a wait the
-    // compiler can see): behind an inline-asm wait it would not know that these loads are complete
-    // and would put its own s_waitcnt vmcnt(0) in front of the first MFMA of the loop body - in
-    // every iteration, draining the ring each time.
-    i32x8 xr[PT][MT][2];
+    // ---- activations: once, into registers, through LDS -------------------------------------------
+    // A lane-per-row load straight into the operand layout touches 16 rows x 64 B per instruction, and the
+    // 16*PT*MT of them a wave needs cost the CU's address unit about 2.6 us in front of the first MFMA
+    // (gate_up at 32 rows: first stage consumed 4.6 us after entry against 1.9 us at 8 rows).  The fragments
+    // therefore take the weights' way: direct-to-LDS loads in the wide pattern (4 rows x 256 B per
+    // instruction), read back with the weight stage's own offsets - which is the operand layout.
+    //
+    // Staging areas of 4 KB (one 16-row block of one K block) per wave: its last ring slot (filled with weights
+    // only afterwards), its share of the reduction scratch (first used at the end of the first tile, behind the
+    // barrier below) and, where the launch has the LDS for it (a.x_extra), one more block behind the scratch.
+    static_assert(MT <= 2, "two staging areas per pass");
+    const unsigned area_lds[3] = {my_ring_lds + (unsigned)(DEPTH - 1) * STAGE_BYTES,
+                                  lds_addr(red) + (unsigned)wave * (2 * FRAGS * 1024),
+                                  lds_addr(red) + (unsigned)(2 * FRAGS * waves + 4 * wave) * 1024};
+    const uint8_t* area_ptr[3] = {my_ring + (size_t)(DEPTH - 1) * STAGE_BYTES,
+                                  reinterpret_cast<const uint8_t*>(red) + (size_t)wave * (2 * FRAGS * 1024),
+                                  reinterpret_cast<const uint8_t*>(red) + (size_t)(2 * FRAGS * waves + 4 * wave) * 1024};
+    auto issue_x = [&](int t, int mt, int area) __attribute__((always_inline)) {
+        const size_t koff = ((size_t)k_block(t) << 8) + src_col;
 #pragma unroll
-    for (int t = 0; t < PT; t++)
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            int row = mt * 16 + r;
+        for (int u = 0; u < 4; u++) {
+            int row = mt * 16 + 4 * u + src_row;
             row = row < a.m ? row : a.m - 1;   // rows past the edge repeat the last one; never stored
-            const uint8_t* src = a.A + (size_t)row * a.k + ((size_t)k_block(t) << 8) + 16 * g;
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const i32x4 lo = __builtin_bit_cast(i32x4, load16(src + (2 * h) * 64));
-                const i32x4 hi = __builtin_bit_cast(i32x4, load16(src + (2 * h + 1) * 64));
-                xr[t][mt][h] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-            }
+            dma_1kb(a.A + (size_t)row * a.k + koff + ((p + u) & 3) * 16, area_lds[area] + u * 1024);
         }
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the activation fragments and the first DEPTH stages
-    asm volatile("" ::: "memory");
+    };
+    i32x8 xr[PT][MT][2];
+    auto read_x = [&](int t, int mt, int area) __attribute__((always_inline)) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(area_ptr[area] + rd_off + (2 * h) * 256);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(area_ptr[area] + rd_off + (2 * h + 1) * 256);
+            xr[t][mt][h] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
+    };
+    constexpr int FIRST = DEPTH - 1;   // weight stages issued before the activations are in registers
+    // Four blocks, three areas: three blocks go in front of the weights, so that their wait leaves the weights in
+    // flight; the fourth - second row block of the wave's second K block - follows as soon as an area is free and
+    // is read in the first tile's second step, which has to wait for the weights issued before it anyway.
+    const bool late_block = MT == 2 && PT == 2 && a.x_extra != 0 && total >= DEPTH + 2;   // wave-uniform
+    int issued = 0;
+    if (late_block) {
+        issue_x(0, 0, 0);
+        issue_x(0, 1 % MT, 1);
+        issue_x(1 % PT, 0, 2);
+        for (; issued < FIRST; issued++) issue(issued);
+        stamps.mark(1);
+        wait_vmcnt<FIRST * PER_STAGE>();
+        read_x(0, 0, 0);
+        read_x(0, 1 % MT, 1);
+        read_x(1 % PT, 0, 2);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // in registers before the areas are written again
+        __syncthreads();   // every wave has what it staged in the reduction scratch
+        issue_x(1 % PT, 1 % MT, 2);
+        issue(issued);
+        issued++;
+    } else {
+        // one K block per pass: the first pass in front of the weights, the others behind them in the queue
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) issue_x(0, mt, mt);
+        for (; issued < FIRST && issued < total; issued++) issue(issued);
+        stamps.mark(1);
+        if (issued == FIRST) wait_vmcnt<FIRST * PER_STAGE>();
+        else wait_vmcnt<0>();
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) read_x(0, mt, mt);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int t = 1; t < PT; t++) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) issue_x(t, mt, mt);
+            wait_vmcnt<0>();
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) read_x(t, mt, mt);
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+        __syncthreads();   // every wave has its fragments: the reduction scratch may be written
+        if (issued < total) {
+            issue(issued);
+            issued++;
+        }
+    }
+    stamps.mark(2);
 
     for (int j = 0; j < my_tiles; j++) {
 #pragma unroll
         for (int t = 0; t < PT; t++) {
             const int i = j * PT + t;
             const int behind = total - 1 - i;   // stages issued after this one, if fewer than DEPTH - 1
-            if (behind >= DEPTH - 1) wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            if (late_block && j == 0) {
+                // behind stage 0: stages 1 .. DEPTH-1 and the late block; behind the late block: stage DEPTH-1 and
+                // the refill of step 0 (total >= DEPTH + 2, so both exist) - with two slots stage 1 is that stage
+                // DEPTH-1, so it is the one to wait for, with only the refill behind it
+                if (t == 0) wait_vmcnt<(DEPTH - 1) * PER_STAGE + 4>();
+                else {
+                    wait_vmcnt<(DEPTH >= 3 ? 2 : 1) * PER_STAGE>();
+                    if (t == 1) {
+                        read_x(1 % PT, 1 % MT, 2);
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    }
+                }
+            } else if (behind >= DEPTH - 1) wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
             else wait_vmcnt_upto(behind * PER_STAGE);
             consume(i, xr[t]);
             // the slot is refilled only after its reads have returned
@@ -186,8 +260,10 @@ __global__ void __launch_bounds__(xreg_launch_bound(MT, RG, PT)) lds_gemm_xreg_k
             if (i + DEPTH < total) issue(i + DEPTH);
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (j == my_tiles - 1) stamps.mark(3);
         tile_done(j);
     }
+    stamps.end(a);
 }
 
 }  // namespace sg
