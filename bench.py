@@ -68,7 +68,7 @@ def main():
                          "times each on cold weights, after three 256 MiB copies of known traffic, and exit "
                          "(for HBM-traffic counter runs; prints no JSON line)")
     ap.add_argument("--sparse-counters", action="store_true",
-                    help="only launch the 2:4 GEMMs (14336 x 4096 and 28672 x 4096 at M = 8, 16), eagerly, three times each "
+                    help="only launch the 2:4 GEMMs (14336 x 4096 and 28672 x 4096 at M = 8, 16; then 4096 x 14336 at M = 8, 16, 32 through the library's choice only), eagerly, three times each "
                          "on cold weights through the library's choice and three times through the one-wave-workgroup kernel "
                          "it replaced, after three 256 MiB copies of known traffic, and exit (for L2 / HBM traffic counter runs; "
                          "prints no JSON line)")
@@ -396,6 +396,29 @@ def main():
                             raise RuntimeError("sg_sparse24_gemm_tuned: %s" % sg.strerror(rc))
                     torch.cuda.synchronize()
             del vb, mb
+        # the long-K shape of the configuration (one 16-row tile per CU): the library's choice at 8, 16 and 32 rows
+        n, k = 4096, 14336
+        copies = 9
+        vb, mb = [], []
+        for _ in range(copies):
+            dense = torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8)
+            v = torch.empty((n, k // 2), device="cuda", dtype=torch.uint8)
+            t = torch.empty((n, k // 8), device="cuda", dtype=torch.uint8)
+            if lib.sg_sparse24_compress(dense.data_ptr(), v.data_ptr(), t.data_ptr(), n, k, k, None) != 0:
+                raise RuntimeError("sg_sparse24_compress failed")
+            vb.append(v)
+            mb.append(t)
+        del dense
+        torch.cuda.synchronize()
+        for j, m in enumerate((8, 16, 32)):
+            a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+            d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+            for i in range(3):
+                rc = lib.sg_sparse24_gemm(a8.data_ptr(), vb[3 * j + i].data_ptr(), mb[3 * j + i].data_ptr(), d.data_ptr(),
+                                          one.data_ptr(), m, n, k, None)
+                if rc != 0:
+                    raise RuntimeError("sg_sparse24_gemm: %s" % sg.strerror(rc))
+            torch.cuda.synchronize()
         return
 
     if args.mid_batch_counters:
