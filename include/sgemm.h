@@ -188,8 +188,13 @@ int sg_skinny_gemm_bf16act_tuned(const void* X_bf16, const uint8_t* B, void* D_b
                                  const SgTuning* tuning, void* stream);
 int sg_skinny_gemm_bf16act_choice(int m, int n, int k, SgTuning* out, int* fused);
 
-/* The configuration sg_skinny_gemm_auto would use, for logging and tuning drivers.
- * out[8] = {split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops}. */
+/* The configuration sg_skinny_gemm_auto would use, in the eight integers of the reference's launcher
+ * (skinny_gemm_caller.cu:55-75), for logging and for drivers written against those:
+ * out[8] = {split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops}.
+ * The eight cannot say everything a launch here depends on (persistent workgroups, resident activations,
+ * the epilogue wave, the mid-batch tiles): passed back through sg_skinny_gemm they select a kernel of the
+ * same ring geometry, not necessarily the one sg_skinny_gemm_auto runs.  sg_skinny_gemm_choice below
+ * returns the complete record, and sg_skinny_gemm_tuned replays exactly that. */
 int sg_skinny_gemm_pick(int m, int n, int k, int out[8]);
 
 /* The complete record sg_skinny_gemm_auto would launch for the shape: the tuning table's entry when
