@@ -658,17 +658,40 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             c.rg = 1;
             c.persist = 1;
             const size_t x_res = (size_t)blocks * xu0 * 1024;
+            if (blocks >= 2 && blocks <= 8) {
+                // a short K: one wave per K block, each with the activation fragments of its block in registers.  Against
+                // the resident-in-LDS kernel on eight waves, some of them without a block, us: 8 x 28672 x 1024 9.7 -> 8.5,
+                // x 512 7.9 -> 7.3, x 1536 10.9 -> 10.4, x 2048 13.0 -> 12.3; 8 x 57344 x 1024 16.0 -> 13.4;
+                // 32 x 28672 x 1024 13.6 -> 9.9.
+                c.waves = blocks;
+                c.depth = blocks <= 2 ? 3 : 2;
+                c.wavetile = 3;
+                return c;
+            }
+            // as many waves (at most eight) as divide the K blocks evenly, so that none idles through part of every
+            // tile: 12 blocks on six waves 16.3 -> 15.9 us (8 x 28672 x 3072), 10 on five 14.9 -> 14.1 (x 2560)
             c.waves = 8;
+            for (int w = 8; w >= 4; w--)
+                if (blocks % w == 0) {
+                    c.waves = w;
+                    break;
+                }
             c.depth = 2;
             if (m <= 16 * c.mt && x_res + (size_t)c.waves * (c.depth * 4 + 2 * c.mt) * 1024 + 4096 <= 159 * 1024) {
                 c.wavetile = 2 | 4;   // resident activations + a dedicated epilogue wave (0.3-0.9 us on gate_up)
                 return c;
             }
             c.waves = m <= 8 ? 8 : 6;
-            if (c.mt == 2 && blocks % 8 == 0 && (blocks / 8) * c.mt <= 4) {
-                // 17..32 rows and a short K: eight waves keep the activation fragments of their own K blocks in registers
-                c.waves = 8;
-                c.depth = 3;
+            // The activations do not fit LDS next to the rings (17..32 rows, or a long K): up to eight waves keep the
+            // fragments of their own K blocks in registers - K = 256 * waves * blocks per wave, at most 4 / m_blocks of
+            // them.  Against what ran before, us: 32 x 28672 x 3072 19.4 -> 17.6 (six waves), x 1024 13.6 -> 9.8 (four),
+            // x 1536 15.3 -> 11.7, x 2560 17.3 -> 15.5, x 3584 20.9 -> 19.7, x 512 12.7 -> 9.0; 16 x 28672 x 8192
+            // 41.5 -> 38.3, 16 x 28672 x 6144 33.0 -> 29.1, 16 x 14336 x 8192 25.3 -> 24.1.
+            for (int w = 8; w >= 2; w--) {
+                const int pt = blocks / w;   // compiled for 1, 2 and 4 blocks per wave
+                if (blocks % w != 0 || pt * c.mt > 4 || pt == 3) continue;
+                c.waves = w;
+                c.depth = blocks / w == 1 ? (w <= 2 ? 4 : 2) : 3;
                 c.wavetile = 3;
                 return c;
             }

@@ -774,3 +774,27 @@ def test_decode_sweep_shapes(sg, oracle, m, n, k):
             torch.cuda.synchronize()
             assert rc == 0, sg.strerror(rc)
             assert oracle.max_rel_err_bf16(bits(D), ref) <= GEMM_TOL, split_k
+
+
+# (m, n, k) -> (waves, wave_tiles) the library chooses for many-tile shapes away from k = 4096: one wave per K
+# block with the activations in registers for a short K, as many waves as divide the K blocks evenly for the
+# resident-in-LDS kernel, registers again where the activations do not fit LDS
+_WIDE_CHOICES = [
+    ((8, 9216, 1024), (4, 3)), ((32, 9216, 1024), (4, 3)), ((8, 9216, 512), (2, 3)), ((20, 9216, 1536), (6, 3)),
+    ((8, 9232, 2048), (8, 3)), ((8, 9216, 3072), (6, 6)), ((16, 9216, 2560), (5, 6)), ((32, 9216, 3072), (6, 3)),
+    ((24, 9216, 3584), (7, 3)), ((16, 8208, 8192), (8, 3)), ((12, 8192 + 16, 6144), (6, 3)), ((3, 9216, 2816), (8, 6)),
+]
+
+
+@pytest.mark.parametrize("shape,choice", _WIDE_CHOICES)
+def test_wide_shapes_with_other_k(sg, oracle, shape, choice):
+    """More than two 16-row tiles per CU and a K other than 4096: the persistent kernels with the wave count the
+    heuristics derive from the number of K blocks, through the library's own choice, against the oracle."""
+    m, n, k = shape
+    t, from_table = sg.skinny_gemm_choice(m, n, k)
+    assert not from_table and t.persistent_wgs_per_cu == 1 and (t.waves, t.wave_tiles) == choice, \
+        (t.waves, t.wave_tiles, t.depth)
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=5)
+    ref = gemm_reference(oracle, a8, b8, scale)
+    got = _run_fast(sg, a8, b8, scale)
+    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL

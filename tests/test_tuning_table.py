@@ -187,7 +187,7 @@ def test_the_heuristics_only_choose_what_the_launchers_take():
     sg.tuning_clear()
     ms = [1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 256, 300, 512]
     ns = [2, 16, 18, 256, 1000, 4096, 4112, 6144, 8192, 10240, 14336, 28672, 57344, 128256]
-    ks = [256, 512, 768, 1024, 2048, 4096, 5120, 8192, 14336, 28672]
+    ks = [256, 512, 768, 1024, 1536, 2048, 2560, 2816, 3072, 3584, 4096, 5120, 6144, 7168, 8192, 10240, 12288, 14336, 28672]
     checked = {1: 0, 2: 0, 4: 0}
     for m in ms:
         for n in ns:

@@ -4,6 +4,8 @@ Its split-K partials and arrival counters live in a fixed array of the library's
 GPU shares and that keeps the last call's contents, so the check is made on two calls in a row, the second on a
 smaller problem, and both against the existing entry point and the CPU oracle.
 """
+import gc
+
 import numpy as np
 import pytest
 import torch
@@ -42,6 +44,10 @@ def test_noalloc_matches_tuned_on_two_calls_in_a_row(sg, oracle, pair):
         got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
         print("case", call, m, n, k, tuning, flush=True)
         assert sg.skinny_gemm_tuned(A, B, want, S, **tuning) == 0
+        # (tensors of earlier tests that the garbage collector has not freed yet must not be freed between the two
+        # readings: collect them first)
+        gc.collect()
+        torch.cuda.synchronize()
         before = torch.cuda.memory_allocated(), sg.workspace_bytes()
         rc = sg.skinny_gemm_tuned_noalloc(A, B, got, S, **tuning)
         assert rc == 0, sg.strerror(rc)
