@@ -133,7 +133,7 @@ def search_space(m, n, k):
         return out
     mb = 1 if m <= 16 else 2
     if k % 256 == 0:
-        for sk, waves, rt, depth, persist, wt in itertools.product((1, 2, 4), (1, 2, 3, 4, 6, 8), (1, 2, 4), (2, 3, 4, 6, 8),
+        for sk, waves, rt, depth, persist, wt in itertools.product((1, 2, 4), (1, 2, 3, 4, 5, 6, 7, 8), (1, 2, 4), (2, 3, 4, 6, 8),
                                                                   (0, 1), (0, 1, 2, 6, 3, 7)):
             if wt and not persist:
                 continue

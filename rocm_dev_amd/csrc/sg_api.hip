@@ -650,7 +650,7 @@ static Config pick_config(int m, int n, int k, int cu_count) {
         c.ku = 4;
         const int blocks = k / 256;
         const int xu0 = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
-        if (c.mt == 2 ? tiles16 >= 2 * cu_count : tiles16 > 2 * cu_count) {
+        if (tiles16 > 2 * cu_count) {
             // more than two tiles per CU (at exactly two, one-wave workgroups are still 2-3 % ahead up to 16 rows;
             // at 2.25 they are 20 % behind): one persistent workgroup per CU walks them with continuous rings;
             // when one activation tile covers all of m, it stays resident in LDS and the stages
@@ -695,11 +695,22 @@ static Config pick_config(int m, int n, int k, int cu_count) {
                 c.wavetile = 3;
                 return c;
             }
-            if (c.mt == 2) {                    // wide tiles share one activation stage among four weight tiles
+            if (c.mt == 2) {
+                // 17..32 rows, activations neither in LDS nor in registers: one workgroup per tile.  Up to three tiles
+                // per CU one-wave workgroups on 16-row tiles (32 x 10240 x 8192 26.5 -> 20.4 us, 32 x 12288 x 5120
+                // 18.0 -> 15.6), above that 64-row tiles, which share an activation stage among four weight tiles, on
+                // three waves (32 x 13824 x 5120 18.3 -> 16.5, 32 x 12288 x 12288 41.7 -> 36.0; 16-row tiles fall off
+                // a cliff there: 26.4)
                 c.persist = 0;
-                c.rg = 4;
-                c.waves = 1;
-                c.depth = 2;
+                if (tiles16 <= 3 * cu_count) {
+                    c.rg = 1;
+                    c.waves = 1;
+                    c.depth = 3;
+                } else {
+                    c.rg = 4;
+                    c.waves = 3;
+                    c.depth = 2;
+                }
                 return c;
             }
             c.depth = 3;
@@ -708,7 +719,11 @@ static Config pick_config(int m, int n, int k, int cu_count) {
                 c.waves--;
             if (c.waves == 5) c.waves = 4;
         } else if (c.mt == 2) {                 // 17..32 activation rows: the activation traffic rivals the weights'
-            if (blocks >= 48) {
+            // (exactly two 16-row tiles per CU belong here: 32-row tiles, one per CU - 32 x 8192 x 8192 23.8 -> 15.0 us
+            // against 64-row tiles on half the CUs, 32 x 8192 x 4096 9.95 -> 9.50 against the register-resident kernel.
+            // A long K is split in two only where that fills the device: with more than one tile per CU the unsplit
+            // 32-row tiles win, 32 x 5120 x 13824 25.5 -> 20.6, 20 x 8192 x 14336 27.9 -> 23.3)
+            if (blocks >= 48 && tiles16 <= cu_count) {
                 c.rg = 2;
                 c.waves = 2;
                 c.depth = 3;
