@@ -747,9 +747,12 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             // workgroups are resident at once); 24-row tiles that give every CU one workgroup level that.  Measured
             // on 6144 x 4096: level with 16-row tiles up to 8 activation rows (6.75 against 6.70 us - the launch is
             // bound by its fixed costs and the stream rate, not by the imbalance), 3-5 % ahead at 9..16 rows
-            // (7.00 against 7.23-7.40 us), where the activation stage is shared by more weight rows.
+            // (7.00 against 7.23-7.40 us), where the activation stage is shared by more weight rows.  With a longer K
+            // a tile is worth more against the fixed costs and the levelling pays at any row count: 8 x 5120 x 5120
+            // 7.8 -> 7.3, 8 x 6144 x 8192 11.1 -> 10.6, 8 x 5120 x 13824 16.7 -> 14.8, 8 x 6144 x 14336 18.7 -> 16.9.
             const int tiles24 = (n + 23) / 24;
-            if (m > 8 && ((tiles24 + cu_count - 1) / cu_count) * 24 < ((tiles16 + cu_count - 1) / cu_count) * 16) {
+            if ((m > 8 || blocks > 16) &&
+                ((tiles24 + cu_count - 1) / cu_count) * 24 < ((tiles16 + cu_count - 1) / cu_count) * 16) {
                 c.rg = 2;
                 c.wavetile = 8;
                 c.waves = 2;
