@@ -850,7 +850,48 @@ static Config config_from_tuning(const SgTuning& t) {
     return c;
 }
 
+// 33..64 activation rows on a small weight matrix: the skinny ring over two 32-row activation tiles (the second
+// tile's weight reads are served by L2: its workgroups run beside the first tile's on the same XCD) beats the
+// mid-batch tiles, which leave most CUs without work or split K to fill them.  Same-process medians, us, against
+// the mid-batch choice: 64 x 4096 x 4096 13.2 -> 9.6, x 2048 8.9 -> 6.5, x 6144 14.6 -> 12.8, x 8192 16.5 -> 15.5;
+// 64 x 2048 x 4096 13.2 -> 7.1, 64 x 2048 x 8192 15.5 -> 10.5, 64 x 1024 x 4096 12.8 -> 6.6, 48 x 3072 x 3072
+// 10.9 -> 7.6; 64 x 5120 x 5120 18.2 -> 15.5, 64 x 4608 x 4096 13.5 -> 12.2.  (From 6144 rows or K = 14336 on the
+// mid-batch engine is level or ahead.)
+static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
+    if (m <= 32 || m > 64 || k % 256 != 0) return false;
+    const int tiles16 = (n + 15) / 16, blocks = k / 256;
+    Config c;
+    c.engine = ENGINE_LDS;
+    c.mt = 2;
+    c.nt = 1;
+    c.ku = 4;
+    c.split_k = 1;
+    c.persist = 0;
+    c.wavetile = 0;
+    if (tiles16 <= cu_count && blocks <= 32) {
+        if (tiles16 * 2 <= cu_count) {   // 16-row tiles: every (tile, activation tile) pair gets a CU
+            c.rg = 1;
+            c.waves = 2;
+            c.depth = 3;
+        } else {                         // 32-row tiles, one workgroup per CU
+            c.rg = 2;
+            c.waves = 2;
+            c.depth = 2;
+        }
+    } else if (tiles16 * 4 <= cu_count * 5 && blocks <= 20) {
+        c.rg = 1;
+        c.waves = 1;
+        c.depth = 3;
+    } else {
+        return false;
+    }
+    *out = c;
+    return true;
+}
+
 static Config heuristic_config(int m, int n, int k, int cu_count) {
+    Config two;
+    if (two_pass_config(m, n, k, cu_count, &two)) return two;
     return (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, cu_count) : pick_config(m, n, k, cu_count);
 }
 

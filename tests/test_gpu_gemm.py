@@ -798,3 +798,23 @@ def test_wide_shapes_with_other_k(sg, oracle, shape, choice):
     ref = gemm_reference(oracle, a8, b8, scale)
     got = _run_fast(sg, a8, b8, scale)
     assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+
+
+@pytest.mark.parametrize("m,n,k,tile_rows", [(33, 4096, 4096, 32), (64, 4096, 4096, 32), (48, 2048, 8192, 16), (64, 1040, 4096, 16),
+                                             (40, 3072, 3072, 32), (64, 5120, 5120, 16), (57, 4608, 2048, 16)])
+def test_two_activation_tiles_on_the_skinny_ring(sg, oracle, m, n, k, tile_rows):
+    """33..64 rows on a small weight matrix: the library's own choice is the skinny LDS ring over two 32-row
+    activation tiles (the second of them partly empty), not the mid-batch engine; against the oracle."""
+    t, from_table = sg.skinny_gemm_choice(m, n, k)
+    assert not from_table and (t.engine, t.m_blocks, 16 * t.row_tiles, t.split_k) == (2, 2, tile_rows, 1)
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=9)
+    ref = gemm_reference(oracle, a8, b8, scale)
+    got = _run_fast(sg, a8, b8, scale)
+    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    # the row/column-scaled entry point goes through the same choice
+    rs = np.random.default_rng(m).uniform(0.5, 2.0, size=m).astype(np.float32)
+    cs = np.random.default_rng(n).uniform(0.5, 2.0, size=n).astype(np.float32)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_rowcol(dev(a8), dev(b8), D, scale_tensor(scale), dev(rs), dev(cs)) == 0
+    torch.cuda.synchronize()
+    assert oracle.max_rel_err_bf16(bits(D), rowcol_reference(oracle, a8, b8, scale, rs, cs)) <= GEMM_TOL
