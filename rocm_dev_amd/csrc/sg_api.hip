@@ -650,6 +650,17 @@ static Config pick_config(int m, int n, int k, int cu_count) {
         c.ku = 4;
         const int blocks = k / 256;
         const int xu0 = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
+        // Fewer 16-row tiles than half the CUs and K of 7168 or more: the idle CUs take K splits, up to four, of at least
+        // 14 K blocks (8 at 17..32 rows) each.  Against one workgroup per tile, us: 8 x 2048 x 14336 10.9 -> 8.6,
+        // 8 x 1024 x 14336 10.6 -> 7.6, 8 x 512 x 28672 18.6 -> 8.9, 16 x 1024 x 8192 7.7 -> 6.8, 8 x 2048 x 8192 7.3 -> 6.9;
+        // 32 x 1024 x 14336 13.1 -> 8.9, 32 x 2048 x 14336 13.8 -> 10.9, 32 x 512 x 28672 20.1 -> 10.9, 32 x 512 x 8192 8.8 -> 7.0.
+        // (At K = 4096 the unsplit launch is ahead: 24 x 2048 x 4096 6.2 against 6.6.)
+        int few_tiles_split = 1;
+        if (tiles16 * 2 <= cu_count && blocks >= 28) {
+            const int per_split = c.mt == 2 ? 8 : 14;
+            few_tiles_split = std::min(std::min(cu_count / tiles16, blocks / per_split), 4);
+            if (few_tiles_split < 2) few_tiles_split = 1;
+        }
         if (tiles16 > 2 * cu_count) {
             // more than two tiles per CU (at exactly two, one-wave workgroups are still 2-3 % ahead up to 16 rows;
             // at 2.25 they are 20 % behind): one persistent workgroup per CU walks them with continuous rings;
@@ -723,7 +734,12 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             // against 64-row tiles on half the CUs, 32 x 8192 x 4096 9.95 -> 9.50 against the register-resident kernel.
             // A long K is split in two only where that fills the device: with more than one tile per CU the unsplit
             // 32-row tiles win, 32 x 5120 x 13824 25.5 -> 20.6, 20 x 8192 x 14336 27.9 -> 23.3)
-            if (blocks >= 48 && tiles16 <= cu_count) {
+            if (few_tiles_split > 1) {          // fewer tiles than half the CUs and a long K: see below
+                c.rg = 1;
+                c.waves = 2;
+                c.depth = 3;
+                c.split_k = few_tiles_split;
+            } else if (blocks >= 48 && tiles16 <= cu_count) {
                 c.rg = 2;
                 c.waves = 2;
                 c.depth = 3;
@@ -743,6 +759,7 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             c.rg = 1;
             c.waves = 1;
             c.depth = 8;
+            c.split_k = few_tiles_split;
             // between one and two 16-row tiles per CU half of the CUs stream twice what the others do (all
             // workgroups are resident at once); 24-row tiles that give every CU one workgroup level that.  Measured
             // on 6144 x 4096: level with 16-row tiles up to 8 activation rows (6.75 against 6.70 us - the launch is
