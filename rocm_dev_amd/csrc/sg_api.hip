@@ -874,9 +874,11 @@ static Config config_from_tuning(const SgTuning& t) {
 // 64 x 2048 x 4096 13.2 -> 7.1, 64 x 2048 x 8192 15.5 -> 10.5, 64 x 1024 x 4096 12.8 -> 6.6, 48 x 3072 x 3072
 // 10.9 -> 7.6; 64 x 5120 x 5120 18.2 -> 15.5, 64 x 4608 x 4096 13.5 -> 12.2.  (From 6144 rows or K = 14336 on the
 // mid-batch engine is level or ahead.)
+// The same holds up to 256 rows while one round of workgroups covers all (weight tile, activation tile) pairs:
+// 128 x 2048 x 4096 13.0 -> 9.9, 128 x 1024 x 4096 12.6 -> 7.3, 256 x 1024 x 4096 12.8 -> 11.0, 96 x 2048 x 8192 15.9 -> 14.5.
 static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
-    if (m <= 32 || m > 64 || k % 256 != 0) return false;
-    const int tiles16 = (n + 15) / 16, blocks = k / 256;
+    if (m <= 32 || m > 256 || k % 256 != 0) return false;
+    const int tiles16 = (n + 15) / 16, blocks = k / 256, m_tiles = (m + 31) / 32;
     Config c;
     c.engine = ENGINE_LDS;
     c.mt = 2;
@@ -885,17 +887,17 @@ static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
     c.split_k = 1;
     c.persist = 0;
     c.wavetile = 0;
-    if (tiles16 <= cu_count && blocks <= 32) {
-        if (tiles16 * 2 <= cu_count) {   // 16-row tiles: every (tile, activation tile) pair gets a CU
+    if (((tiles16 + 1) / 2) * m_tiles <= cu_count && blocks <= 32) {
+        if (tiles16 * m_tiles <= cu_count) {   // 16-row tiles: every (tile, activation tile) pair gets a CU
             c.rg = 1;
             c.waves = 2;
             c.depth = 3;
-        } else {                         // 32-row tiles, one workgroup per CU
+        } else {                               // 32-row tiles, at most one workgroup per CU
             c.rg = 2;
             c.waves = 2;
             c.depth = 2;
         }
-    } else if (tiles16 * 4 <= cu_count * 5 && blocks <= 20) {
+    } else if (m <= 64 && tiles16 * 4 <= cu_count * 5 && blocks <= 20) {
         c.rg = 1;
         c.waves = 1;
         c.depth = 3;

@@ -801,10 +801,11 @@ def test_wide_shapes_with_other_k(sg, oracle, shape, choice):
 
 
 @pytest.mark.parametrize("m,n,k,tile_rows", [(33, 4096, 4096, 32), (64, 4096, 4096, 32), (48, 2048, 8192, 16), (64, 1040, 4096, 16),
-                                             (40, 3072, 3072, 32), (64, 5120, 5120, 16), (57, 4608, 2048, 16)])
+                                             (40, 3072, 3072, 32), (64, 5120, 5120, 16), (57, 4608, 2048, 16),
+                                             (128, 2048, 4096, 32), (100, 1024, 4096, 16), (256, 1024, 2048, 32), (96, 2048, 8192, 32)])
 def test_two_activation_tiles_on_the_skinny_ring(sg, oracle, m, n, k, tile_rows):
-    """33..64 rows on a small weight matrix: the library's own choice is the skinny LDS ring over two 32-row
-    activation tiles (the second of them partly empty), not the mid-batch engine; against the oracle."""
+    """More than 32 rows on a small weight matrix: the library's own choice is the skinny LDS ring over several 32-row
+    activation tiles (the last of them partly empty), not the mid-batch engine; against the oracle."""
     t, from_table = sg.skinny_gemm_choice(m, n, k)
     assert not from_table and (t.engine, t.m_blocks, 16 * t.row_tiles, t.split_k) == (2, 2, tile_rows, 1)
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=9)
