@@ -724,11 +724,19 @@ static Config pick_config(int m, int n, int k, int cu_count) {
                 }
                 return c;
             }
-            c.depth = 3;
-            c.waves = 6;
-            while (c.waves > 2 && (size_t)c.waves * (c.depth * (4 + xu0) + 2 * c.mt) * 1024 + 4096 > 159 * 1024)
-                c.waves--;
-            if (c.waves == 5) c.waves = 4;
+            // Up to 16 rows, the activations neither in LDS nor in registers (a long K that the waves cannot divide):
+            // 9..16 rows share an activation stage among four weight tiles, 64-row tiles on two waves (16 x 14336 x 14336
+            // 41.2 -> 32.5 us, 16 x 28672 x 10240 57.2 -> 47.4 against six waves on 16-row tiles); up to 8 rows one
+            // workgroup of four waves per 16-row tile (8 x 28672 x 14336 63.8 -> 60.4, 4 x 57344 x 14336 120 -> 115).
+            if (m > 8) {
+                c.rg = 4;
+                c.waves = 2;
+                c.depth = 2;
+            } else {
+                c.persist = 0;
+                c.waves = 4;
+                c.depth = 3;
+            }
         } else if (c.mt == 2) {                 // 17..32 activation rows: the activation traffic rivals the weights'
             // (exactly two 16-row tiles per CU belong here: 32-row tiles, one per CU - 32 x 8192 x 8192 23.8 -> 15.0 us
             // against 64-row tiles on half the CUs, 32 x 8192 x 4096 9.95 -> 9.50 against the register-resident kernel.
