@@ -130,6 +130,12 @@ def search_space(m, n, k):
             r = record(ENGINE_MID, sk, waves, rt, mb, depth, dx if dx else depth)
             if mid_fits(k, r):
                 out.append(r)
+        # the skinny LDS ring over several 32-row activation tiles (what the library runs on small weight matrices)
+        if m <= 256 and k % 256 == 0:
+            for sk, waves, rt, depth in itertools.product((1, 2), (1, 2, 3, 4), (1, 2, 4), (2, 3, 4)):
+                r = record(ENGINE_LDS, sk, waves, rt, 2, depth, 4, 1, 0, 0)
+                if lds_ring_fits(m, k, r):
+                    out.append(r)
         return out
     mb = 1 if m <= 16 else 2
     if k % 256 == 0:

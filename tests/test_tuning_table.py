@@ -128,7 +128,8 @@ def test_search_space_respects_the_fit_rules():
     # the library's own choices for the benchmark shapes are inside the space
     import rocm_dev_amd as sg
     sg.tuning_clear()
-    for (m, n, k) in [(8, 28672, 4096), (8, 4096, 4096), (32, 28672, 4096), (16, 4096, 14336)]:
+    for (m, n, k) in [(8, 28672, 4096), (8, 4096, 4096), (32, 28672, 4096), (16, 4096, 14336), (64, 4096, 4096), (128, 1024, 4096),
+                      (8, 28672, 3072), (32, 28672, 1536), (16, 28672, 8192), (32, 10240, 8192), (8, 1024, 14336)]:
         choice, _ = sg.skinny_gemm_choice(m, n, k)
         assert autotune_fields(choice) in autotune.search_space(m, n, k), (m, n, k, autotune_fields(choice))
     # every k the library takes has candidates, down to a single partial 64-byte stage
@@ -138,8 +139,13 @@ def test_search_space_respects_the_fit_rules():
     # a k the LDS ring cannot take (not a multiple of 256) gets direct-engine candidates only
     assert {r["engine"] for r in autotune.search_space(8, 4096, 4096 + 64)} == {autotune.ENGINE_DIRECT}
     # mid-batch: the ring must fit 160 KB; 256 x 256 tiles only with a shallow activation ring
-    mid = autotune.search_space(256, 57344, 8192)
-    assert mid and all(r["engine"] == autotune.ENGINE_MID and autotune.mid_fits(8192, r) for r in mid)
+    space = autotune.search_space(256, 57344, 8192)
+    mid = [r for r in space if r["engine"] == autotune.ENGINE_MID]
+    assert mid and all(autotune.mid_fits(8192, r) for r in mid)
+    # ... next to them the skinny ring over several 32-row activation tiles, one workgroup per tile
+    rest = [r for r in space if r["engine"] != autotune.ENGINE_MID]
+    assert rest and all(r["engine"] == autotune.ENGINE_LDS and r["m_blocks"] == 2 and r["persistent_wgs_per_cu"] == 0
+                        and autotune.lds_ring_fits(256, 8192, r) for r in rest)
     big = [r for r in mid if r["waves"] == 8 and r["row_tiles"] == 4 and r["m_blocks"] == 8]
     assert big and all((r["depth"], r["k_chunks"]) in ((2, 2), (3, 2)) for r in big)
     for shape in [(256, 57344, 8192), (128, 8192, 8192), (64, 8192, 28672), (64, 10240, 8192)]:
