@@ -798,6 +798,13 @@ def test_wide_shapes_with_other_k(sg, oracle, shape, choice):
     ref = gemm_reference(oracle, a8, b8, scale)
     got = _run_fast(sg, a8, b8, scale)
     assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+    # per-row and per-column factors through the same kernels
+    rs = np.random.default_rng(k).uniform(0.5, 2.0, size=m).astype(np.float32)
+    cs = np.random.default_rng(n).uniform(0.5, 2.0, size=n).astype(np.float32)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_rowcol(dev(a8), dev(b8), D, scale_tensor(scale), dev(rs), dev(cs)) == 0
+    torch.cuda.synchronize()
+    assert oracle.max_rel_err_bf16(bits(D), rowcol_reference(oracle, a8, b8, scale, rs, cs)) <= GEMM_TOL
 
 
 @pytest.mark.parametrize("m,n,k,tile_rows", [(33, 4096, 4096, 32), (64, 4096, 4096, 32), (48, 2048, 8192, 16), (64, 1040, 4096, 16),
