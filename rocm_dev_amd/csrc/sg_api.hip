@@ -669,14 +669,31 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             c.rg = 1;
             c.persist = 1;
             const size_t x_res = (size_t)blocks * xu0 * 1024;
-            if (blocks >= 2 && blocks <= 8) {
-                // a short K: one wave per K block, each with the activation fragments of its block in registers.  Against
-                // the resident-in-LDS kernel on eight waves, some of them without a block, us: 8 x 28672 x 1024 9.7 -> 8.5,
-                // x 512 7.9 -> 7.3, x 1536 10.9 -> 10.4, x 2048 13.0 -> 12.3; 8 x 57344 x 1024 16.0 -> 13.4;
-                // 32 x 28672 x 1024 13.6 -> 9.9.
-                c.waves = blocks;
-                c.depth = blocks <= 2 ? 3 : 2;
-                c.wavetile = 3;
+            if (blocks <= 10) {
+                // a short K: every wave owns whole tiles over all of K - no reduction across waves in front of the
+                // store - next to the whole activation matrix in LDS (at most 80 KB), eight waves x two slots.  Against
+                // one wave per K block with its activation fragments in registers, us, cold weights: 8 x 28672 x 256
+                // 8.5 -> 3.8, x 512 7.2 -> 4.9, x 1024 8.4 -> 7.3, x 2048 13.1 -> 11.7, x 2560 15.0 -> 14.0;
+                // 16 x 57344 x 1024 13.5 -> 12.4, 32 x 28672 x 1024 9.8 -> 8.1, x 2048 14.4 -> 12.7, x 2560 17.1 -> 15.0,
+                // 24 x 28672 x 512 8.8 -> 5.5.  (From 12 K blocks on the K-split waves below are level or ahead.)
+                c.waves = 8;
+                c.depth = 2;
+                c.wavetile = 1;
+                if (tiles16 <= 4 * cu_count) {
+                    // up to four tiles per CU eight waves do not all find a tile: four waves x four slots at 17..32 rows
+                    // (32 x 10240 x 2048 7.75 -> 6.67, 32 x 9216 x 2560 8.74 -> 7.36, 24 x 16384 x 2560 10.9 -> 10.1),
+                    // and one-wave workgroups per tile up to 16 rows from 1024 columns of K on, 2-5 % ahead of that
+                    // (8 x 16384 x 1024 5.29 -> 5.03, x 2048 7.71 -> 7.29, 16 x 16384 x 2048 7.73 -> 7.57)
+                    if (c.mt == 2) {
+                        c.waves = 4;
+                        c.depth = 4;
+                    } else if (blocks >= 4) {
+                        c.persist = 0;
+                        c.wavetile = 0;
+                        c.waves = 1;
+                        c.depth = 3;
+                    }
+                }
                 return c;
             }
             // as many waves (at most eight) as divide the K blocks evenly, so that none idles through part of every
@@ -695,9 +712,8 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             c.waves = m <= 8 ? 8 : 6;
             // The activations do not fit LDS next to the rings (17..32 rows, or a long K): up to eight waves keep the
             // fragments of their own K blocks in registers - K = 256 * waves * blocks per wave, at most 4 / m_blocks of
-            // them.  Against what ran before, us: 32 x 28672 x 3072 19.4 -> 17.6 (six waves), x 1024 13.6 -> 9.8 (four),
-            // x 1536 15.3 -> 11.7, x 2560 17.3 -> 15.5, x 3584 20.9 -> 19.7, x 512 12.7 -> 9.0; 16 x 28672 x 8192
-            // 41.5 -> 38.3, 16 x 28672 x 6144 33.0 -> 29.1, 16 x 14336 x 8192 25.3 -> 24.1.
+            // them.  Against what ran before, us: 32 x 28672 x 3072 19.4 -> 17.6 (six waves), x 3584 20.9 -> 19.7;
+            // 16 x 28672 x 8192 41.5 -> 38.3, 16 x 28672 x 6144 33.0 -> 29.1, 16 x 14336 x 8192 25.3 -> 24.1.
             for (int w = 8; w >= 2; w--) {
                 const int pt = blocks / w;   // compiled for 1, 2 and 4 blocks per wave
                 if (blocks % w != 0 || pt * c.mt > 4 || pt == 3) continue;

@@ -780,20 +780,24 @@ def test_decode_sweep_shapes(sg, oracle, m, n, k):
 # block with the activations in registers for a short K, as many waves as divide the K blocks evenly for the
 # resident-in-LDS kernel, registers again where the activations do not fit LDS
 _WIDE_CHOICES = [
-    ((8, 9216, 1024), (4, 3)), ((32, 9216, 1024), (4, 3)), ((8, 9216, 512), (2, 3)), ((20, 9216, 1536), (6, 3)),
-    ((8, 9232, 2048), (8, 3)), ((8, 9216, 3072), (6, 6)), ((16, 9216, 2560), (5, 6)), ((32, 9216, 3072), (6, 3)),
-    ((24, 9216, 3584), (7, 3)), ((16, 8208, 8192), (8, 3)), ((12, 8192 + 16, 6144), (6, 3)), ((3, 9216, 2816), (8, 6)),
+    # shape, (persistent workgroups per CU, waves, wave_tiles) of the library's own choice
+    ((8, 9216, 1024), (0, 1, 0)), ((32, 9216, 1024), (1, 4, 1)), ((8, 9216, 512), (1, 8, 1)), ((20, 9216, 1536), (1, 4, 1)),
+    ((8, 9232, 2048), (0, 1, 0)), ((8, 9216, 3072), (1, 6, 6)), ((16, 9216, 2560), (0, 1, 0)), ((32, 9216, 3072), (1, 6, 3)),
+    ((24, 9216, 3584), (1, 7, 3)), ((16, 8208, 8192), (1, 8, 3)), ((12, 8192 + 16, 6144), (1, 6, 3)), ((3, 9216, 2816), (1, 8, 6)),
+    ((8, 20480 + 16, 1024), (1, 8, 1)), ((16, 24576, 2560), (1, 8, 1)), ((5, 20480, 256), (1, 8, 1)), ((32, 9216, 256), (1, 4, 1)),
+    ((27, 12288 + 8, 2560), (1, 4, 1)), ((32, 20480, 2048), (1, 8, 1)), ((13, 16400, 2048), (1, 8, 1)),
 ]
 
 
 @pytest.mark.parametrize("shape,choice", _WIDE_CHOICES)
 def test_wide_shapes_with_other_k(sg, oracle, shape, choice):
-    """More than two 16-row tiles per CU and a K other than 4096: the persistent kernels with the wave count the
-    heuristics derive from the number of K blocks, through the library's own choice, against the oracle."""
+    """More than two 16-row tiles per CU and a K other than 4096: whole tiles per wave next to resident activations
+    for a short K (one-wave workgroups per tile up to four tiles per CU), otherwise the persistent kernels with the
+    wave count the heuristics derive from the number of K blocks; through the library's own choice, against the oracle."""
     m, n, k = shape
     t, from_table = sg.skinny_gemm_choice(m, n, k)
-    assert not from_table and t.persistent_wgs_per_cu == 1 and (t.waves, t.wave_tiles) == choice, \
-        (t.waves, t.wave_tiles, t.depth)
+    assert not from_table and (t.persistent_wgs_per_cu, t.waves, t.wave_tiles) == choice, \
+        (t.persistent_wgs_per_cu, t.waves, t.wave_tiles, t.depth)
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=5)
     ref = gemm_reference(oracle, a8, b8, scale)
     got = _run_fast(sg, a8, b8, scale)
