@@ -215,7 +215,7 @@ class Bench:
         self.torch = torch
         self.m, self.n, self.k = m, n, k
         g = torch.Generator(device="cuda").manual_seed(seed)
-        rot = max(2, int(640e6 // (n * k)) + 1)
+        rot = min(96, max(2, int(640e6 // (n * k)) + 1))
         # codes 0..119 and 128..247: finite E4M3 of both signs up to 240
         def codes(rows):
             c = torch.randint(0, 120, (rows, k), dtype=torch.uint8, device="cuda", generator=g)
@@ -233,8 +233,10 @@ class Bench:
 
     def time(self, lib, tuning, launches=20, repeats=3):
         """Microseconds per launch, best of `repeats` replays of a graph of `launches` back-to-back launches
-        over the weight rotation; None if the library rejects the record."""
+        over the weight rotation (at least one launch per buffer: a replay must not find the previous replay's
+        weights in the last-level cache); None if the library rejects the record."""
         torch = self.torch
+        launches = max(launches, len(self.weights))
         if self.launch(lib, tuning, self.weights[0], torch.cuda.current_stream().cuda_stream) != 0:
             return None
         torch.cuda.synchronize()
