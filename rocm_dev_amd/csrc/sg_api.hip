@@ -446,7 +446,10 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     struct Tile { int bn, bm, waves; };
     // {224, *, 14}: fourteen waves; 57344 = 256 x 224 gives every CU a tile where 256-row tiles fill 224 of 256
     // (5-10 % at M = 128 and 256 on N(0,1)-quantised operands, 4 % at M = 64 over two co-resident 128 x 64 tiles)
-    static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4}, {256, 128, 8}, {224, 128, 14},
+    // (a 64 x 128 tile on four waves was in this list; wherever the rounds rule chose it - 129..192 or more than 256
+    // rows on a narrow weight matrix, where its padded rows look like a fuller round - 128 x 64 on eight waves measured
+    // 6-12 % faster, ten shapes)
+    static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {256, 128, 8}, {224, 128, 14},
                                  {256, 64, 8}, {224, 64, 14}, {128, 256, 8}, {256, 256, 8}, {224, 256, 14}};
     const int bm_max = m <= 64 ? 64 : (m <= 128 ? 128 : 256);
     const int blocks = k / 128;
@@ -454,21 +457,34 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     long best_rounds = -1, best_wgs = 0;
     for (const Tile& t : order) {
         if (t.bm > bm_max) continue;
-        const long tiles = (long)((n + t.bn - 1) / t.bn) * ((m + t.bm - 1) / t.bm);
+        const long m_tiles = (m + t.bm - 1) / t.bm;
+        const long tiles = (long)((n + t.bn - 1) / t.bn) * m_tiles;
         for (int sk = 1; sk <= 4; sk++) {
             // a three-way split only up to 64 activation rows, where the partials are small against the weights
             // (64 x 10240 x 8192: 80 tiles -> 240 workgroups, 24.5 -> 22.5 us); two and four ways keep 32 K blocks
             if (sk == 3 ? (m > 64 || blocks / sk < 16) : (sk > 1 && blocks / sk < 32)) continue;
+            // the fp32 partials of a split are written and read back: no split whose partials (padded rows x 4 bytes x
+            // splits per weight row) exceed a third of the weight row's k bytes (320 x 8192 x 8192: 256-row tiles split
+            // in two 51.9 us, 128-row tiles unsplit 39.3)
+            if (sk > 1 && m_tiles * t.bm * 4 * sk * 3 > k) continue;
             const long wgs = tiles * sk;
             const long rounds = (wgs + cu_count - 1) / cu_count;
-            // the fourteen-wave tile only where it is known to pay: unsplit, one tile covering all of m (the
-            // weights streamed once), and exactly filling its rounds
-            if (t.waves == 14 && (sk > 1 || m > t.bm || n % t.bn != 0 || wgs % cu_count != 0)) continue;
-            const bool better = best_rounds < 0 || rounds < best_rounds ||
-                                (rounds == best_rounds && wgs * 16 > best_wgs * 17) ||   // clearly fuller round
-                                // as full with less splitting, when the splits had become short
-                                (rounds == best_rounds && wgs == best_wgs && sk < best.split_k &&
-                                 blocks / best.split_k < 48);
+            // the fourteen-wave tile only where it is known to pay: unsplit, exactly filling its rounds, and all of m
+            // in one tile or tiles of at least 128 rows (the weights streamed at most a few times: 144..256 x 28672 x
+            // 4096 on two 224 x 128 tiles 3-4 % ahead of 256 x 128, 320 and 448 rows on 224 x 256 11-15 % ahead of 256 x 256)
+            if (t.waves == 14 && (sk > 1 || (m > t.bm && t.bm < 128) || n % t.bn != 0 || wgs % cu_count != 0)) continue;
+            bool better = best_rounds < 0 || rounds < best_rounds ||
+                          (rounds == best_rounds && wgs * 16 > best_wgs * 17) ||   // clearly fuller round
+                          // as full with less splitting, when the splits had become short
+                          (rounds == best_rounds && wgs == best_wgs && sk < best.split_k &&
+                           blocks / best.split_k < 48);
+            if (best_rounds >= 0 && rounds == best_rounds && blocks < 96 && m > 64) {
+                // above 64 rows and below K = 12288 an unsplit launch that fills 70 % of its rounds beats a split one
+                // that fills them all (144 x 8192 x 8192: 192 workgroups unsplit 29.1 us, 256 split in two 31.7);
+                // with a longer K the split wins (448 x 4096 x 14336: 46.2 against 50.4)
+                if (sk == 1 && best.split_k > 1 && wgs * 10 >= rounds * cu_count * 7) better = true;
+                if (sk > 1 && best.split_k == 1 && best_wgs * 10 >= rounds * cu_count * 7) better = false;
+            }
             if (!better) continue;
             best_rounds = rounds;
             best_wgs = wgs;

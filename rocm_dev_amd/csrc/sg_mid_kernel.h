@@ -83,8 +83,32 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     const int wn = wave % WN, wm = wave / WN;
     const bool loads_x = XW == WAVES || wave < XW;   // wave-uniform
 
+    // Workgroups go to the eight XCDs round-robin by id, and each XCD has its own L2.  The workgroups that share a
+    // weight tile (its activation tiles and K splits) take consecutive slots of ONE XCD, so the tile crosses the
+    // fabric once and its readers run side by side: position j in an order that lists the weight tiles of XCD 0
+    // (tile_n = 0, 8, 16 ...), then XCD 1's, each with all of its workgroups, and XCD x starting where its
+    // share of the grid starts.  Tile counts that 8 does not divide put at most a few tiles on two XCDs.
     int tile_n, split, tile_m;
-    decode_tile(a, (int)blockIdx.x, tile_n, split, tile_m);
+    {
+        const int bid = (int)blockIdx.x, grid = (int)gridDim.x;
+        const int xcd = bid & 7, qs = grid >> 3, rs = grid & 7;
+        const int j = xcd * qs + (xcd < rs ? xcd : rs) + (bid >> 3);
+        const int per_tile = a.split_k * a.m_tiles;
+        const int r = j / per_tile, p = j - r * per_tile;
+        const int qn = a.n_tiles >> 3, rn = a.n_tiles & 7;
+        int g, i;
+        if (r < rn * (qn + 1)) {
+            g = r / (qn + 1);
+            i = r - g * (qn + 1);
+        } else {                                 // (reached only with qn > 0: otherwise every r is below rn)
+            const int r2 = r - rn * (qn + 1);
+            g = rn + r2 / qn;
+            i = r2 - (g - rn) * qn;
+        }
+        tile_n = g + 8 * i;
+        split = p / a.m_tiles;
+        tile_m = p - split * a.m_tiles;
+    }
     const int n0 = tile_n * BN;
     const int m0 = tile_m * BM;
 

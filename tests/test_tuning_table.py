@@ -174,10 +174,14 @@ def test_heuristics_pick_the_fourteen_wave_tile_where_it_fills_the_chip():
         assert not from_table
         got = (t.engine, t.split_k, t.waves, t.row_tiles, t.m_blocks, t.depth, t.k_chunks if t.k_chunks else t.depth)
         assert got == (autotune.ENGINE_MID, 1, 14, 2, mb, depth, dx), (m, got)
-    # a row count that 224 does not divide, or more rows than one tile covers: eight-wave tiles as before
-    for m, n in ((64, 57344 + 128), (300, 57344)):
+    # a row count that 224 does not divide: eight-wave tiles as before
+    t, _ = api.skinny_gemm_choice(64, 57344 + 128, 8192)
+    assert t.waves != 14
+    # more rows than one tile covers: tiles of 128 rows or more still fill every round (two 224 x 256 tiles per CU, two
+    # 224 x 128 tiles on half as many weight rows), 64-row tiles are not stacked
+    for m, n, mb in ((300, 57344, 8), (448, 28672, 8), (200, 28672, 4)):
         t, _ = api.skinny_gemm_choice(m, n, 8192)
-        assert t.waves != 14, (m, n)
+        assert (t.engine, t.split_k, t.waves, t.m_blocks) == (autotune.ENGINE_MID, 1, 14, mb), (m, n)
 
 
 def test_the_heuristics_only_choose_what_the_launchers_take():
