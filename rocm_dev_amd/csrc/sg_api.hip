@@ -446,17 +446,20 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     struct Tile { int bn, bm, waves; };
     // {224, *, 14}: fourteen waves; 57344 = 256 x 224 gives every CU a tile where 256-row tiles fill 224 of 256
     // (5-10 % at M = 128 and 256 on N(0,1)-quantised operands, 4 % at M = 64 over two co-resident 128 x 64 tiles)
-    // (a 64 x 128 tile on four waves was in this list; wherever the rounds rule chose it - 129..192 or more than 256
-    // rows on a narrow weight matrix, where its padded rows look like a fuller round - 128 x 64 on eight waves measured
-    // 6-12 % faster, ten shapes)
-    static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {256, 128, 8}, {224, 128, 14},
+    // The 64 x 128 tile on four waves only where it covers all of m and K is beyond 4096 (stacked - 129..192 or more
+    // than 256 rows on a narrow weight matrix, where its padded rows look like a fuller round - 128 x 64 on eight waves
+    // measured 6-12 % faster, ten shapes).
+    static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4}, {256, 128, 8}, {224, 128, 14},
                                  {256, 64, 8}, {224, 64, 14}, {128, 256, 8}, {256, 256, 8}, {224, 256, 14}};
     const int bm_max = m <= 64 ? 64 : (m <= 128 ? 128 : 256);
     const int blocks = k / 128;
     Config best;
     long best_rounds = -1, best_wgs = 0;
+    const Tile* best_tile = nullptr;
     for (const Tile& t : order) {
         if (t.bm > bm_max) continue;
+        const bool tall4 = t.bn == 64 && t.bm == 128;
+        if (tall4 && (m > 128 || blocks <= 32)) continue;
         const long m_tiles = (m + t.bm - 1) / t.bm;
         const long tiles = (long)((n + t.bn - 1) / t.bn) * m_tiles;
         for (int sk = 1; sk <= 4; sk++) {
@@ -469,10 +472,11 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
             if (sk > 1 && m_tiles * t.bm * 4 * sk * 3 > k) continue;
             const long wgs = tiles * sk;
             const long rounds = (wgs + cu_count - 1) / cu_count;
-            // the fourteen-wave tile only where it is known to pay: unsplit, exactly filling its rounds, and all of m
-            // in one tile or tiles of at least 128 rows (the weights streamed at most a few times: 144..256 x 28672 x
-            // 4096 on two 224 x 128 tiles 3-4 % ahead of 256 x 128, 320 and 448 rows on 224 x 256 11-15 % ahead of 256 x 256)
-            if (t.waves == 14 && (sk > 1 || (m > t.bm && t.bm < 128) || n % t.bn != 0 || wgs % cu_count != 0)) continue;
+            // the fourteen-wave tile only where it is known to pay: unsplit, filling at least 70 % of its rounds, and all
+            // of m in one tile or tiles of at least 128 rows (the weights streamed at most a few times: 144..256 x 28672 x
+            // 4096 on two 224 x 128 tiles 3-4 % ahead of 256 x 128, 320 and 448 rows on 224 x 256 11-15 % ahead of
+            // 256 x 256; 448 x 13824 x 5120, 62 tiles x 4, 52.3 -> 47.4)
+            if (t.waves == 14 && (sk > 1 || (m > t.bm && t.bm < 128) || wgs * 10 < rounds * cu_count * 7)) continue;
             bool better = best_rounds < 0 || rounds < best_rounds ||
                           (rounds == best_rounds && wgs * 16 > best_wgs * 17) ||   // clearly fuller round
                           // as full with less splitting, when the splits had become short
@@ -485,9 +489,17 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
                 if (sk == 1 && best.split_k > 1 && wgs * 10 >= rounds * cu_count * 7) better = true;
                 if (sk > 1 && best.split_k == 1 && best_wgs * 10 >= rounds * cu_count * 7) better = false;
             }
+            // 65..128 rows, K beyond 4096: against 128 x 64 on eight waves and two activation tiles, one 64 x 128 tile
+            // over all of m on four waves - as many workgroups, the weights pass each CU once (72 x 13824 x 5120
+            // 29.6 -> 23.5 us, 100 rows 28.6 -> 26.1, 72 x 14336 x 5120 28.3 -> 23.7, 72 x 12288 x 5120 28.0 -> 23.0;
+            // level at K = 4096)
+            if (tall4 && sk == 1 && rounds == best_rounds && best_tile && best_tile->bn == 128 && best_tile->bm == 64 &&
+                best.split_k == 1 && wgs * 16 >= best_wgs * 15)
+                better = true;
             if (!better) continue;
             best_rounds = rounds;
             best_wgs = wgs;
+            best_tile = &t;
             best.waves = t.waves;
             best.rg = t.bn / (t.waves * 8);      // 16-row tiles per wave: bn = 16 * rg * (waves / 2)
             best.mt = t.bm / 32;

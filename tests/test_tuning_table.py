@@ -184,6 +184,22 @@ def test_heuristics_pick_the_fourteen_wave_tile_where_it_fills_the_chip():
         assert (t.engine, t.split_k, t.waves, t.m_blocks) == (autotune.ENGINE_MID, 1, 14, mb), (m, n)
 
 
+def test_mid_batch_tile_choice_between_the_tile_heights():
+    """Row counts that no tile height divides: padded rows are not a fuller round (no stacked 64 x 128 tiles), a split
+    whose fp32 partials rival the weights is not taken, an unsplit round that is 70 % full stays unsplit below
+    K = 12288, one 64 x 128 tile covers 65..128 rows when K is beyond 4096, and fourteen-wave tiles of 128 rows or more
+    may be stacked.  (tile n, tile m, waves, split) per shape, as measured best or within 2 % of it."""
+    want = {(160, 8192, 8192): (128, 64, 8, 1), (144, 6144, 4096): (128, 64, 8, 1), (320, 8192, 8192): (128, 128, 8, 1),
+            (144, 4096, 14336): (128, 64, 8, 2), (448, 4096, 14336): (128, 128, 8, 2), (320, 4096, 4096): (128, 64, 8, 1),
+            (72, 13824, 5120): (64, 128, 4, 1), (72, 14336, 4096): (128, 64, 8, 1), (448, 13824, 5120): (224, 128, 14, 1),
+            (200, 28672, 4096): (224, 128, 14, 1), (448, 28672, 8192): (224, 256, 14, 1), (128, 8192, 8192): (64, 64, 4, 1)}
+    for (m, n, k), tile in want.items():
+        t, from_table = api.skinny_gemm_choice(m, n, k)
+        assert not from_table and t.engine == autotune.ENGINE_MID
+        got = (8 * t.row_tiles * t.waves, 32 * t.m_blocks, t.waves, t.split_k)
+        assert got == tile, ((m, n, k), got)
+
+
 def test_the_heuristics_only_choose_what_the_launchers_take():
     """A sweep of shapes through the library's own choice (no table): whatever engine it names, the record must be one
     the launch rules - written down independently of the launchers - accept, so a legal shape cannot fail in the
