@@ -434,6 +434,17 @@ def main():
                         raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
                 torch.cuda.synchronize()
             del wb
+        # stacked activation tiles on weight tile counts that 8 (the XCDs) does not divide, or over more than one round
+        for (m, n, k) in ((288, 11008, 4096), (448, 13824, 5120), (320, 22016, 4096), (200, 28672, 8192)):
+            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(2)]
+            a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+            d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+            for i in range(3):
+                rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % 2].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, None)
+                if rc != 0:
+                    raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
+            torch.cuda.synchronize()
+            del wb
         return
 
     from rocm_dev_amd import synth
