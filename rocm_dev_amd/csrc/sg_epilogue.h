@@ -77,13 +77,19 @@ inline void set_reciprocals(StreamArgs& a) {
     a.inv_waves = div_reciprocal((unsigned)a.waves);
 }
 
-// Position `bid` in tile order -> (tile_n, split, tile_m): n tiles fastest, then the K splits of a tile, then m tiles.
+// Position `bid` in tile order -> (tile_n, split, tile_m): the activation tiles of a weight tile fastest (their
+// workgroups are neighbours in position, hence - after xcd_order - on one XCD, whose L2 then fetches the weight tile
+// once for all of them), then the n tiles, then the K splits.  With one activation tile this is n tiles fastest.
 __device__ __forceinline__ void decode_tile(const StreamArgs& a, int bid, int& tile_n, int& split, int& tile_m) {
-    const unsigned q = fast_div((unsigned)bid, (unsigned)a.n_tiles, a.inv_n_tiles);
-    tile_n = bid - (int)q * a.n_tiles;
-    const unsigned m = fast_div(q, (unsigned)a.split_k, a.inv_split_k);
-    split = (int)(q - m * (unsigned)a.split_k);
-    tile_m = (int)m;
+    unsigned rest = (unsigned)bid;
+    tile_m = 0;
+    if (a.m_tiles > 1) {
+        rest = (unsigned)bid / (unsigned)a.m_tiles;
+        tile_m = bid - (int)rest * a.m_tiles;
+    }
+    const unsigned q = fast_div(rest, (unsigned)a.n_tiles, a.inv_n_tiles);
+    tile_n = (int)rest - (int)q * a.n_tiles;
+    split = (int)q;
 }
 
 // K range [b_begin, b_end) of split `split` out of `blocks` stage-sized blocks; the last split takes the remainder.
