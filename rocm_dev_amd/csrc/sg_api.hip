@@ -919,18 +919,22 @@ static Config config_from_tuning(const SgTuning& t) {
     return c;
 }
 
-// 33..64 activation rows on a small weight matrix: the skinny ring over two 32-row activation tiles (the second
-// tile's weight reads are served by L2: its workgroups run beside the first tile's on the same XCD) beats the
-// mid-batch tiles, which leave most CUs without work or split K to fill them.  Same-process medians, us, against
-// the mid-batch choice: 64 x 4096 x 4096 13.2 -> 9.6, x 2048 8.9 -> 6.5, x 6144 14.6 -> 12.8, x 8192 16.5 -> 15.5;
-// 64 x 2048 x 4096 13.2 -> 7.1, 64 x 2048 x 8192 15.5 -> 10.5, 64 x 1024 x 4096 12.8 -> 6.6, 48 x 3072 x 3072
-// 10.9 -> 7.6; 64 x 5120 x 5120 18.2 -> 15.5, 64 x 4608 x 4096 13.5 -> 12.2.  (From 6144 rows or K = 14336 on the
-// mid-batch engine is level or ahead.)
-// The same holds up to 256 rows while one round of workgroups covers all (weight tile, activation tile) pairs:
-// 128 x 2048 x 4096 13.0 -> 9.9, 128 x 1024 x 4096 12.6 -> 7.3, 256 x 1024 x 4096 12.8 -> 11.0, 96 x 2048 x 8192 15.9 -> 14.5.
+// 33..256 activation rows on a small weight matrix: the skinny ring over several 32-row activation tiles beats the
+// mid-batch tiles, which leave most CUs without work or split K to fill them, as long as one round of workgroups
+// covers every (weight tile, activation tile) pair.  The activation tiles of a weight tile are neighbours in tile
+// order, i.e. on one XCD, whose L2 fetches the weight tile once for all of them.  The smallest weight tile - 16, 32 or
+// 64 rows - that fits the round; 64-row tiles only up to K = 5120 (level at 8192, behind at 14336).  Same-process
+// medians, us, cold weights, against the mid-batch choice: 64 x 1024 x 4096 12.7 -> 5.9, 128 x 2048 x 4096 12.8 -> 7.2,
+// 256 x 1024 x 4096 12.4 -> 6.7, 64 x 4096 x 4096 13.3 -> 8.0, 128 x 4096 x 4096 13.1 -> 10.9, 256 x 2048 x 4096
+// 12.7 -> 10.2, 64 x 8192 x 4096 14.2 -> 12.2, 128 x 4096 x 2048 8.7 -> 7.4, 96 x 5120 x 5120 16.1 -> 13.5,
+// 128 x 2048 x 8192 16.6 -> 10.7, 64 x 4096 x 8192 16.6 -> 12.6, 128 x 2048 x 14336 23.8 -> 17.1, 64 x 2048 x 14336
+// 20.4 -> 13.5.  Up to 64 rows one-wave workgroups on 16-row tiles still win at up to one and a half tiles per CU
+// (64 x 6144 x 4096 13.6 -> 11.0, 64 x 5120 x 5120 18.1 -> 13.4); beyond (64 x 10240 x 4096, 96 x 6144 x 4096,
+// 192 x 4096 x 4096) the mid-batch engine is 10-25 % ahead.
 static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
     if (m <= 32 || m > 256 || k % 256 != 0) return false;
-    const int tiles16 = (n + 15) / 16, blocks = k / 256, m_tiles = (m + 31) / 32;
+    const long tiles16 = (n + 15) / 16, tiles32 = (n + 31) / 32, tiles64 = (n + 63) / 64;
+    const int blocks = k / 256, m_tiles = (m + 31) / 32;
     Config c;
     c.engine = ENGINE_LDS;
     c.mt = 2;
@@ -939,20 +943,21 @@ static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
     c.split_k = 1;
     c.persist = 0;
     c.wavetile = 0;
-    if (((tiles16 + 1) / 2) * m_tiles <= cu_count && blocks <= 32) {
-        if (tiles16 * m_tiles <= cu_count) {   // 16-row tiles: every (tile, activation tile) pair gets a CU
-            c.rg = 1;
-            c.waves = 2;
-            c.depth = 3;
-        } else {                               // 32-row tiles, at most one workgroup per CU
-            c.rg = 2;
-            c.waves = 2;
-            c.depth = 2;
-        }
-    } else if (m <= 64 && tiles16 * 4 <= cu_count * 5 && blocks <= 20) {
+    c.depth = 2;
+    if (tiles16 * m_tiles <= cu_count) {           // 16-row tiles: every (tile, activation tile) pair gets a CU
         c.rg = 1;
+        c.waves = 2;
+        c.depth = 3;
+    } else if (tiles32 * m_tiles <= cu_count) {    // 32-row tiles
+        c.rg = 2;
+        c.waves = blocks > 32 ? 3 : 4;
+    } else if (m <= 64 && tiles16 * 2 <= cu_count * 3 && blocks <= 20) {
+        c.rg = 1;                                  // (2-4 % ahead of 64-row tiles there: 64 x 6144 x 4096 11.0 against 11.5)
         c.waves = 1;
         c.depth = 3;
+    } else if (tiles64 * m_tiles <= cu_count && blocks <= 20) {
+        c.rg = 4;
+        c.waves = 3;
     } else {
         return false;
     }

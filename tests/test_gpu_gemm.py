@@ -813,10 +813,13 @@ def test_wide_shapes_with_other_k(sg, oracle, shape, choice):
 
 @pytest.mark.parametrize("m,n,k,tile_rows", [(33, 4096, 4096, 32), (64, 4096, 4096, 32), (48, 2048, 8192, 16), (64, 1040, 4096, 16),
                                              (40, 3072, 3072, 32), (64, 5120, 5120, 16), (57, 4608, 2048, 16),
-                                             (128, 2048, 4096, 32), (100, 1024, 4096, 16), (256, 1024, 2048, 32), (96, 2048, 8192, 32)])
+                                             (128, 2048, 4096, 32), (100, 1024, 4096, 16), (256, 1024, 2048, 32), (96, 2048, 8192, 32),
+                                             (128, 4096, 4096, 64), (192, 2048, 4096, 64), (64, 8192, 4096, 64), (64, 6144, 4096, 16),
+                                             (128, 2048, 14336, 32), (250, 2000, 5120, 64)])
 def test_two_activation_tiles_on_the_skinny_ring(sg, oracle, m, n, k, tile_rows):
     """More than 32 rows on a small weight matrix: the library's own choice is the skinny LDS ring over several 32-row
-    activation tiles (the last of them partly empty), not the mid-batch engine; against the oracle."""
+    activation tiles (the last of them partly empty) and the smallest weight tile that fits one round of workgroups,
+    not the mid-batch engine; against the oracle."""
     t, from_table = sg.skinny_gemm_choice(m, n, k)
     assert not from_table and (t.engine, t.m_blocks, 16 * t.row_tiles, t.split_k) == (2, 2, tile_rows, 1)
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=9)
@@ -829,4 +832,6 @@ def test_two_activation_tiles_on_the_skinny_ring(sg, oracle, m, n, k, tile_rows)
     D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     assert sg.skinny_gemm_rowcol(dev(a8), dev(b8), D, scale_tensor(scale), dev(rs), dev(cs)) == 0
     torch.cuda.synchronize()
-    assert oracle.max_rel_err_bf16(bits(D), rowcol_reference(oracle, a8, b8, scale, rs, cs)) <= GEMM_TOL
+    # (against the model of the matrix instruction's summation: with these factors the sequential host sum itself lies
+    # 0.0104 from it in one of the 524,288 outputs of 128 x 4096 x 4096, whichever kernel runs)
+    assert oracle.max_rel_err_bf16(bits(D), rowcol_reference(oracle, a8, b8, scale, rs, cs, model=True)) <= GEMM_TOL
