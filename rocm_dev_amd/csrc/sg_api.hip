@@ -923,7 +923,8 @@ static Config config_from_tuning(const SgTuning& t) {
 // mid-batch tiles, which leave most CUs without work or split K to fill them, as long as one round of workgroups
 // covers every (weight tile, activation tile) pair.  The activation tiles of a weight tile are neighbours in tile
 // order, i.e. on one XCD, whose L2 fetches the weight tile once for all of them.  The smallest weight tile - 16, 32 or
-// 64 rows - that fits the round; 64-row tiles only up to K = 5120 (level at 8192, behind at 14336).  Same-process
+// 64 rows - that fits the round; 64-row tiles only below K = 8192 (224 x 1536 x 6144 16.1 -> 12.6; level at 8192, behind
+// at 14336).  Same-process
 // medians, us, cold weights, against the mid-batch choice: 64 x 1024 x 4096 12.7 -> 5.9, 128 x 2048 x 4096 12.8 -> 7.2,
 // 256 x 1024 x 4096 12.4 -> 6.7, 64 x 4096 x 4096 13.3 -> 8.0, 128 x 4096 x 4096 13.1 -> 10.9, 256 x 2048 x 4096
 // 12.7 -> 10.2, 64 x 8192 x 4096 14.2 -> 12.2, 128 x 4096 x 2048 8.7 -> 7.4, 96 x 5120 x 5120 16.1 -> 13.5,
@@ -955,7 +956,7 @@ static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
         c.rg = 1;                                  // (2-4 % ahead of 64-row tiles there: 64 x 6144 x 4096 11.0 against 11.5)
         c.waves = 1;
         c.depth = 3;
-    } else if (tiles64 * m_tiles <= cu_count && blocks <= 20) {
+    } else if (tiles64 * m_tiles <= cu_count && blocks < 32) {
         c.rg = 4;
         c.waves = 3;
     } else {

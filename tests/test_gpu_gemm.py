@@ -815,7 +815,7 @@ def test_wide_shapes_with_other_k(sg, oracle, shape, choice):
                                              (40, 3072, 3072, 32), (64, 5120, 5120, 16), (57, 4608, 2048, 16),
                                              (128, 2048, 4096, 32), (100, 1024, 4096, 16), (256, 1024, 2048, 32), (96, 2048, 8192, 32),
                                              (128, 4096, 4096, 64), (192, 2048, 4096, 64), (64, 8192, 4096, 64), (64, 6144, 4096, 16),
-                                             (128, 2048, 14336, 32), (250, 2000, 5120, 64)])
+                                             (128, 2048, 14336, 32), (250, 2000, 5120, 64), (224, 1536, 6144, 64)])
 def test_two_activation_tiles_on_the_skinny_ring(sg, oracle, m, n, k, tile_rows):
     """More than 32 rows on a small weight matrix: the library's own choice is the skinny LDS ring over several 32-row
     activation tiles (the last of them partly empty) and the smallest weight tile that fits one round of workgroups,
