@@ -264,8 +264,13 @@ static unsigned level_persistent_grid(unsigned tiles, size_t most) {
     return (unsigned)((tiles + rounds - 1) / rounds);
 }
 
+// k of 256 j + 128 (j >= 1) also runs on the per-tile ring: the last block is loaded from k - 256 and half used
+// (the persistent kernels and the kernels that keep the activations resident take multiples of 256 only).
+static bool lds_half_block_k(int k) { return k % 256 == 128 && k > 256; }
+
 static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
-    if (a.k % 256 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (a.k % 256 != 0 && !(lds_half_block_k(a.k) && c.persist == 0 && (c.wavetile & 7) == 0 && !a.A16))
+        return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     // wave_tiles bit 3: 24-row tiles (two fragments, the second half used), one workgroup per tile
     const bool rows24 = (c.wavetile & 8) != 0;
     if (rows24 && (c.rg != 2 || c.mt != 1 || c.persist != 0 || (c.wavetile & 7) != 0)) return SG_INVALID_CONFIG;
@@ -673,10 +678,12 @@ static Config pick_config(int m, int n, int k, int cu_count) {
     c.persist = 0;
     c.wavetile = 0;
     const int tiles16 = (n + 15) / 16;
-    if (k % 256 == 0) {
+    // (a K with half a block at its end only where the per-tile ring runs, up to two tiles per CU: against the
+    // register-streaming engine, us: 8 x 8192 x 29568 58.1 -> 37, 32 x 8192 x 29568 87.9 -> 45, 8 x 2048 x 1408 4.2 -> 3.2)
+    if (k % 256 == 0 || (lds_half_block_k(k) && tiles16 <= 2 * cu_count)) {
         c.engine = ENGINE_LDS;
         c.ku = 4;
-        const int blocks = k / 256;
+        const int blocks = (k + 255) / 256;
         const int xu0 = c.mt == 2 ? 8 : ((m + 3) / 4 <= 1 ? 1 : ((m + 3) / 4 <= 2 ? 2 : 4));
         // Fewer 16-row tiles than half the CUs and K of 7168 or more: the idle CUs take K splits, up to four, of at least
         // 14 K blocks (8 at 17..32 rows) each.  Against one workgroup per tile, us: 8 x 2048 x 14336 10.9 -> 8.6,

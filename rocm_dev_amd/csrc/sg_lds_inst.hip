@@ -15,13 +15,15 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
     if (threads > (unsigned)bound) return SG_INVALID_CONFIG;
     void (*kernel)(const StreamArgs) = nullptr;
     if constexpr (MODE == 4) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true, true>;
-    else if constexpr (MODE == 5) kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
+    else if constexpr (MODE == 5) kernel = (a.k & 255) ? lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true, true>
+                                                        : lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
     else if constexpr (MODE == 2) kernel = lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
     else if constexpr (MODE == 3) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
     else if constexpr (MODE == 1) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false>;
-    else kernel = lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
-    static LdsGranted granted;
-    if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
+    else kernel = (a.k & 255) ? lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false, true>   // half a block at the end of K
+                              : lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
+    static LdsGranted granted[2];
+    if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted[(a.k & 255) ? 1 : 0])) return rc;
     kernel<<<dim3(grid), dim3(threads), lds, stream>>>(a);
     return report_hip("lds_gemm_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }

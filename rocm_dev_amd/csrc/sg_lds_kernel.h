@@ -85,6 +85,17 @@ __device__ __forceinline__ void drain_ring(Consume& consume, int i) {
     consume(i + D);
     if constexpr (D + 1 < DEPTH) drain_ring<D + 1, DEPTH, PER_STAGE>(consume, i);
 }
+// ... with another consumer for the very last stage (the one that may be a half block)
+template <int D, int DEPTH, int PER_STAGE, class Consume, class ConsumeLast>
+__device__ __forceinline__ void drain_ring(Consume& consume, ConsumeLast& consume_last, int i) {
+    wait_vmcnt<(DEPTH - 1 - D) * PER_STAGE>();
+    if constexpr (D + 1 < DEPTH) {
+        consume(i + D);
+        drain_ring<D + 1, DEPTH, PER_STAGE>(consume, consume_last, i);
+    } else {
+        consume_last(i + D);
+    }
+}
 
 
 // One 256-byte K block of a stage: weights at w (16*RG rows, 4 KB per 16-row tile), activations
@@ -117,6 +128,28 @@ __device__ __forceinline__ void mma_block_256(const uint8_t* w, const uint8_t* x
         }
 }
 
+// The last 128 bytes of a K that is 128 beyond a multiple of 256: the stage was loaded from K - 256 (a window that
+// ends with the row, so nothing past it is read) and its first half has been consumed as the second half of the block
+// before - only the second v_mfma of mma_block_256 runs.
+template <int MT, int RG>
+__device__ __forceinline__ void mma_block_second_half(const uint8_t* w, const uint8_t* x, f32x4 (&acc)[RG][MT]) {
+    i32x8 xv[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) {
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(x + mt * 4096 + 2 * 256);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(x + mt * 4096 + 3 * 256);
+        xv[mt] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    }
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(w + rg * 4096 + 2 * 256);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(w + rg * 4096 + 3 * 256);
+        const i32x8 wv = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[rg][mt] = mfma_e4m3_16x16x128(wv, xv[mt], acc[rg][mt]);
+    }
+}
+
 // Tiles of a persistent workgroup: one contiguous run (not a stride of gridDim.x), runs in XCD order.
 struct TileRun { int first, count; };
 __device__ __forceinline__ TileRun persistent_tile_run(int total_tiles) {
@@ -137,7 +170,9 @@ constexpr int lds_persistent_launch_bound(int MT, int RG) { return RG * MT >= 4 
 // HALF2 (RG == 2 only): 24-row tiles - the second 16-row fragment holds 8 weight rows, its other 8 are never fetched
 // (the MFMA reads whatever lies there) and never stored.  6144 rows are 256 tiles of 24 where they are 384 of 16: one
 // workgroup per CU instead of one and a half.
-template <int MT, int RG, int XU, int DEPTH, bool NT, bool HALF2 = false>
+// TAIL: k = 256 j + 128 - the last K block is loaded from k - 256 and only its second half multiplied (a build of its
+// own, so that the loop for whole blocks stays as it is).
+template <int MT, int RG, int XU, int DEPTH, bool NT, bool HALF2 = false, bool TAIL = false>
 __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
     __shared__ unsigned arrival;
@@ -162,9 +197,15 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     const int m0 = tile_m * (16 * MT);
 
     // K range of this workgroup in 256-byte blocks; the last split takes the remainder
+    // (k may be 128 beyond a multiple of 256: the last block is then loaded from k - 256 and half used)
     int b_begin, b_end;
-    split_range(a, a.k >> 8, split, b_begin, b_end);
+    const int blocks_total = (a.k + 255) >> 8;
+    split_range(a, blocks_total, split, b_begin, b_end);
     const int mine = blocks_of_wave(a, b_end - b_begin, wave);
+    int tail_i = -1;                  // which of this wave's stages is the half block, if any: its last one
+    if constexpr (TAIL) {
+        if (b_end == blocks_total && mine > 0 && b_begin + wave + (mine - 1) * waves == blocks_total - 1) tail_i = mine - 1;
+    }
 
     // ---- DMA sources: a wave-uniform base per operand (the tile's first row, advanced along K with scalar
     // adds) plus a 32-bit offset per lane and instruction (the host keeps 64 rows of either operand below 2 GB)
@@ -199,7 +240,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
 
     const size_t k_step = (size_t)waves << 8;
     auto issue = [&](int i) __attribute__((always_inline)) {  // i-th stage of this wave -> slot i % DEPTH
-        const size_t koff = (size_t)i * k_step;
+        const size_t koff = (size_t)i * k_step - ((TAIL && i == tail_i) ? 128 : 0);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
@@ -223,6 +264,11 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
         mma_block_256<MT, RG>(slot, slot + W_INSTR * 1024, acc);
     };
+    auto consume_last = [&](int i) __attribute__((always_inline)) {   // this wave's last stage: whole or half
+        const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
+        if (TAIL && i == tail_i) mma_block_second_half<MT, RG>(slot, slot + W_INSTR * 1024, acc);
+        else mma_block_256<MT, RG>(slot, slot + W_INSTR * 1024, acc);
+    };
 
     if (mine >= DEPTH) {
 #pragma unroll
@@ -240,13 +286,19 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
             issue(i + DEPTH);
             __builtin_amdgcn_sched_barrier(0);
         }
-        drain_ring<0, DEPTH, PER_STAGE>(consume, i);
+        if constexpr (TAIL) drain_ring<0, DEPTH, PER_STAGE>(consume, consume_last, i);
+        else drain_ring<0, DEPTH, PER_STAGE>(consume, i);
     } else {
         for (int i = 0; i < mine; i++) issue(i);
         stamps.mark(1);
         wait_vmcnt<0>();
         stamps.mark(2);
-        for (int i = 0; i < mine; i++) consume(i);
+        if constexpr (TAIL) {
+            for (int i = 0; i + 1 < mine; i++) consume(i);
+            if (mine > 0) consume_last(mine - 1);
+        } else {
+            for (int i = 0; i < mine; i++) consume(i);
+        }
     }
 
     // the ring is reused for the cross-wave reduction: every wave must be done reading it
