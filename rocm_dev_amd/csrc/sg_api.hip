@@ -264,9 +264,9 @@ static unsigned level_persistent_grid(unsigned tiles, size_t most) {
     return (unsigned)((tiles + rounds - 1) / rounds);
 }
 
-// k of 256 j + 128 (j >= 1) also runs on the per-tile ring: the last block is loaded from k - 256 and half used
-// (the persistent kernels and the kernels that keep the activations resident take multiples of 256 only).
-static bool lds_half_block_k(int k) { return k % 256 == 128 && k > 256; }
+// k of 256 j + 64, 128 or 192 (j >= 1) also runs on the per-tile ring: the last block is loaded from k - 256 and
+// partly used (the persistent kernels and the kernels that keep the activations resident take multiples of 256 only).
+static bool lds_half_block_k(int k) { return k % 256 != 0 && k % 64 == 0 && k > 256; }
 
 static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     if (a.k % 256 != 0 && !(lds_half_block_k(a.k) && c.persist == 0 && (c.wavetile & 7) == 0 && !a.A16))
@@ -680,7 +680,7 @@ static Config pick_config(int m, int n, int k, int cu_count) {
     const int tiles16 = (n + 15) / 16;
     // (a K with half a block at its end only where the per-tile ring runs, up to two tiles per CU: against the
     // register-streaming engine, us: 8 x 8192 x 29568 58.1 -> 37, 32 x 8192 x 29568 87.9 -> 45, 8 x 2048 x 1408 4.2 -> 3.2)
-    if (k % 256 == 0 || (lds_half_block_k(k) && tiles16 <= 2 * cu_count)) {
+    if (k % 256 == 0 || (lds_half_block_k(k) && m <= 32 && tiles16 <= 2 * cu_count)) {
         c.engine = ENGINE_LDS;
         c.ku = 4;
         const int blocks = (k + 255) / 256;

@@ -128,25 +128,33 @@ __device__ __forceinline__ void mma_block_256(const uint8_t* w, const uint8_t* x
         }
 }
 
-// The last 128 bytes of a K that is 128 beyond a multiple of 256: the stage was loaded from K - 256 (a window that
-// ends with the row, so nothing past it is read) and its first half has been consumed as the second half of the block
-// before - only the second v_mfma of mma_block_256 runs.
+// The last block of a K that is 64, 128 or 192 beyond a multiple of 256: the stage was loaded from K - 256 (a window
+// that ends with the row, so nothing past it is read) and its first `first_chunk` 64-byte chunks have been consumed
+// with the block before.  A v_mfma whose two chunks are both old is left out; where only its first chunk is old, the
+// activation operand's half for that chunk is zero (the products vanish whatever the weights are - unless a weight
+// is NaN, which had poisoned its column with the block before already).
 template <int MT, int RG>
-__device__ __forceinline__ void mma_block_second_half(const uint8_t* w, const uint8_t* x, f32x4 (&acc)[RG][MT]) {
-    i32x8 xv[MT];
+__device__ __forceinline__ void mma_block_tail(const uint8_t* w, const uint8_t* x, f32x4 (&acc)[RG][MT], int first_chunk) {
 #pragma unroll
-    for (int mt = 0; mt < MT; mt++) {
-        const i32x4 lo = *reinterpret_cast<const i32x4*>(x + mt * 4096 + 2 * 256);
-        const i32x4 hi = *reinterpret_cast<const i32x4*>(x + mt * 4096 + 3 * 256);
-        xv[mt] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    }
+    for (int h = 0; h < 2; h++) {
+        if (2 * h + 1 < first_chunk) continue;            // wave-uniform
+        const bool lo_old = 2 * h < first_chunk;
+        i32x8 xv[MT];
 #pragma unroll
-    for (int rg = 0; rg < RG; rg++) {
-        const i32x4 lo = *reinterpret_cast<const i32x4*>(w + rg * 4096 + 2 * 256);
-        const i32x4 hi = *reinterpret_cast<const i32x4*>(w + rg * 4096 + 3 * 256);
-        const i32x8 wv = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        for (int mt = 0; mt < MT; mt++) {
+            i32x4 lo = *reinterpret_cast<const i32x4*>(x + mt * 4096 + (2 * h) * 256);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(x + mt * 4096 + (2 * h + 1) * 256);
+            if (lo_old) lo = i32x4{0, 0, 0, 0};
+            xv[mt] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        }
 #pragma unroll
-        for (int mt = 0; mt < MT; mt++) acc[rg][mt] = mfma_e4m3_16x16x128(wv, xv[mt], acc[rg][mt]);
+        for (int rg = 0; rg < RG; rg++) {
+            const i32x4 lo = *reinterpret_cast<const i32x4*>(w + rg * 4096 + (2 * h) * 256);
+            const i32x4 hi = *reinterpret_cast<const i32x4*>(w + rg * 4096 + (2 * h + 1) * 256);
+            const i32x8 wv = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) acc[rg][mt] = mfma_e4m3_16x16x128(wv, xv[mt], acc[rg][mt]);
+        }
     }
 }
 
@@ -170,8 +178,8 @@ constexpr int lds_persistent_launch_bound(int MT, int RG) { return RG * MT >= 4 
 // HALF2 (RG == 2 only): 24-row tiles - the second 16-row fragment holds 8 weight rows, its other 8 are never fetched
 // (the MFMA reads whatever lies there) and never stored.  6144 rows are 256 tiles of 24 where they are 384 of 16: one
 // workgroup per CU instead of one and a half.
-// TAIL: k = 256 j + 128 - the last K block is loaded from k - 256 and only its second half multiplied (a build of its
-// own, so that the loop for whole blocks stays as it is).
+// TAIL: k = 256 j + 64, 128 or 192 - the last K block is loaded from k - 256 and only its new chunks multiplied (a
+// build of its own, so that the loop for whole blocks stays as it is).
 template <int MT, int RG, int XU, int DEPTH, bool NT, bool HALF2 = false, bool TAIL = false>
 __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
@@ -197,7 +205,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     const int m0 = tile_m * (16 * MT);
 
     // K range of this workgroup in 256-byte blocks; the last split takes the remainder
-    // (k may be 128 beyond a multiple of 256: the last block is then loaded from k - 256 and half used)
+    // (k may be 64, 128 or 192 beyond a multiple of 256: the last block is then loaded from k - 256 and partly used)
     int b_begin, b_end;
     const int blocks_total = (a.k + 255) >> 8;
     split_range(a, blocks_total, split, b_begin, b_end);
@@ -240,7 +248,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
 
     const size_t k_step = (size_t)waves << 8;
     auto issue = [&](int i) __attribute__((always_inline)) {  // i-th stage of this wave -> slot i % DEPTH
-        const size_t koff = (size_t)i * k_step - ((TAIL && i == tail_i) ? 128 : 0);
+        const size_t koff = (size_t)i * k_step - ((TAIL && i == tail_i) ? (size_t)(256 - (a.k & 255)) : 0);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
@@ -266,7 +274,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     };
     auto consume_last = [&](int i) __attribute__((always_inline)) {   // this wave's last stage: whole or half
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
-        if (TAIL && i == tail_i) mma_block_second_half<MT, RG>(slot, slot + W_INSTR * 1024, acc);
+        if (TAIL && i == tail_i) mma_block_tail<MT, RG>(slot, slot + W_INSTR * 1024, acc, 4 - ((a.k & 255) >> 6));
         else mma_block_256<MT, RG>(slot, slot + W_INSTR * 1024, acc);
     };
 
