@@ -55,7 +55,7 @@ def lds_ring_fits(m, k, r):
     """The LDS-ring kernels' resource rules for one record: ring + resident activations + reduction
     scratch within LDS, and no more DMA instructions in flight than a wave can count."""
     xu = _activation_instructions(m, r["m_blocks"])
-    if k % 256 and not (k % 64 == 0 and k > 256 and not r["persistent_wgs_per_cu"] and not r["wave_tiles"] & 7):
+    if k % 256 and not (k % 16 == 0 and k > 256 and not r["persistent_wgs_per_cu"] and not r["wave_tiles"] & 7):
         return False              # part of a block at the end of K: only the kernel with one workgroup per tile
     blocks = k // 256
     if r["wave_tiles"] & 8:     # 24-row tiles: two fragments, six weight instructions per stage, one workgroup per tile
@@ -140,7 +140,7 @@ def search_space(m, n, k):
                     out.append(r)
         return out
     mb = 1 if m <= 16 else 2
-    if k % 256 == 0 or (k % 64 == 0 and k > 256):
+    if k % 256 == 0 or (k % 16 == 0 and k > 256):
         for sk, waves, rt, depth, persist, wt in itertools.product((1, 2, 4), (1, 2, 3, 4, 5, 6, 7, 8), (1, 2, 4), (2, 3, 4, 6, 8),
                                                                   (0, 1), (0, 1, 2, 6, 3, 7)):
             if wt and not persist:

@@ -264,9 +264,10 @@ static unsigned level_persistent_grid(unsigned tiles, size_t most) {
     return (unsigned)((tiles + rounds - 1) / rounds);
 }
 
-// k of 256 j + 64, 128 or 192 (j >= 1) also runs on the per-tile ring: the last block is loaded from k - 256 and
-// partly used (the persistent kernels and the kernels that keep the activations resident take multiples of 256 only).
-static bool lds_half_block_k(int k) { return k % 256 != 0 && k % 64 == 0 && k > 256; }
+// Any k beyond 256 (a multiple of 16, like every k the library takes) also runs on the per-tile ring: the last block
+// is loaded from k - 256 and partly used (the persistent kernels and the kernels that keep the activations resident
+// take multiples of 256 only).
+static bool lds_half_block_k(int k) { return k % 256 != 0 && k % 16 == 0 && k > 256; }
 
 static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
     if (a.k % 256 != 0 && !(lds_half_block_k(a.k) && c.persist == 0 && (c.wavetile & 7) == 0 && !a.A16))

@@ -128,23 +128,29 @@ __device__ __forceinline__ void mma_block_256(const uint8_t* w, const uint8_t* x
         }
 }
 
-// The last block of a K that is 64, 128 or 192 beyond a multiple of 256: the stage was loaded from K - 256 (a window
-// that ends with the row, so nothing past it is read) and its first `first_chunk` 64-byte chunks have been consumed
-// with the block before.  A v_mfma whose two chunks are both old is left out; where only its first chunk is old, the
-// activation operand's half for that chunk is zero (the products vanish whatever the weights are - unless a weight
-// is NaN, which had poisoned its column with the block before already).
+// The last block of a K that is not a multiple of 256 (but of 16, and beyond 256): the stage was loaded from K - 256
+// (a window that ends with the row, so nothing past it is read) and its first `old_bytes` = 256 - K % 256 bytes have been
+// consumed with the block before.  A v_mfma whose two 64-byte chunks are both old is left out; elsewhere the old part
+// of the activation operand is zero - whole chunks, and in the chunk the boundary runs through the 16-byte pieces
+// below it: lane (r, g) holds piece g of every chunk (the DMA's rotation and the read offset cancel), so that is a
+// per-lane select.  The products vanish whatever the weights are - unless a weight is NaN, which had poisoned its
+// column with the block before already.
 template <int MT, int RG>
-__device__ __forceinline__ void mma_block_tail(const uint8_t* w, const uint8_t* x, f32x4 (&acc)[RG][MT], int first_chunk) {
+__device__ __forceinline__ void mma_block_tail(const uint8_t* w, const uint8_t* x, f32x4 (&acc)[RG][MT], int old_bytes, int g) {
+    const int first_chunk = old_bytes >> 6, first_piece = (old_bytes & 63) >> 4;   // wave-uniform
+    const bool piece_old = g < first_piece;                                        // per lane
 #pragma unroll
     for (int h = 0; h < 2; h++) {
-        if (2 * h + 1 < first_chunk) continue;            // wave-uniform
-        const bool lo_old = 2 * h < first_chunk;
+        if (2 * h + 1 < first_chunk) continue;
+        const bool lo_old = 2 * h < first_chunk || (2 * h == first_chunk && piece_old);
+        const bool hi_old = 2 * h + 1 == first_chunk && piece_old;
         i32x8 xv[MT];
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
             i32x4 lo = *reinterpret_cast<const i32x4*>(x + mt * 4096 + (2 * h) * 256);
-            const i32x4 hi = *reinterpret_cast<const i32x4*>(x + mt * 4096 + (2 * h + 1) * 256);
+            i32x4 hi = *reinterpret_cast<const i32x4*>(x + mt * 4096 + (2 * h + 1) * 256);
             if (lo_old) lo = i32x4{0, 0, 0, 0};
+            if (hi_old) hi = i32x4{0, 0, 0, 0};
             xv[mt] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
         }
 #pragma unroll
@@ -178,8 +184,8 @@ constexpr int lds_persistent_launch_bound(int MT, int RG) { return RG * MT >= 4 
 // HALF2 (RG == 2 only): 24-row tiles - the second 16-row fragment holds 8 weight rows, its other 8 are never fetched
 // (the MFMA reads whatever lies there) and never stored.  6144 rows are 256 tiles of 24 where they are 384 of 16: one
 // workgroup per CU instead of one and a half.
-// TAIL: k = 256 j + 64, 128 or 192 - the last K block is loaded from k - 256 and only its new chunks multiplied (a
-// build of its own, so that the loop for whole blocks stays as it is).
+// TAIL: k not a multiple of 256 - the last K block is loaded from k - 256 and only its new bytes multiplied (a build of
+// its own, so that the loop for whole blocks stays as it is).
 template <int MT, int RG, int XU, int DEPTH, bool NT, bool HALF2 = false, bool TAIL = false>
 __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
@@ -205,7 +211,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     const int m0 = tile_m * (16 * MT);
 
     // K range of this workgroup in 256-byte blocks; the last split takes the remainder
-    // (k may be 64, 128 or 192 beyond a multiple of 256: the last block is then loaded from k - 256 and partly used)
+    // (k need not be a multiple of 256: the last block is then loaded from k - 256 and partly used)
     int b_begin, b_end;
     const int blocks_total = (a.k + 255) >> 8;
     split_range(a, blocks_total, split, b_begin, b_end);
@@ -274,7 +280,7 @@ __global__ void __launch_bounds__(lds_launch_bound(MT, RG)) lds_gemm_kernel(cons
     };
     auto consume_last = [&](int i) __attribute__((always_inline)) {   // this wave's last stage: whole or half
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
-        if (TAIL && i == tail_i) mma_block_tail<MT, RG>(slot, slot + W_INSTR * 1024, acc, 4 - ((a.k & 255) >> 6));
+        if (TAIL && i == tail_i) mma_block_tail<MT, RG>(slot, slot + W_INSTR * 1024, acc, 256 - (a.k & 255), g);
         else mma_block_256<MT, RG>(slot, slot + W_INSTR * 1024, acc);
     };
 

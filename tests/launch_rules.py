@@ -27,9 +27,8 @@ def expect_lds(m, n, k, r):
     waves, rg, mt, depth, sk = r["waves"], r["row_tiles"], r["m_blocks"], r["depth"], r["split_k"]
     persist, wt = r["persistent_wgs_per_cu"], r["wave_tiles"]
     if k % 256:
-        # part of a block at the end of K (64, 128 or 192 bytes): only the kernel with one workgroup per tile (16-, 32-,
-        # 64- or 24-row tiles)
-        if not (k % 64 == 0 and k > 256 and persist == 0 and wt & 7 == 0):
+        # part of a block at the end of K: only the kernel with one workgroup per tile (16-, 32-, 64- or 24-row tiles)
+        if not (k % 16 == 0 and k > 256 and persist == 0 and wt & 7 == 0):
             return 3
     blocks = k // 256
     if not (1 <= waves <= 16 and depth >= 1 and rg >= 1 and mt in (1, 2) and 1 <= sk <= blocks):

@@ -135,7 +135,8 @@ LDS_CONFIGS = [
                                    (32, 512, 2048), (27, 100, 1280), (40, 64, 512),
                                    # part of a 256-byte block at the end of K (loaded from k - 256, the new chunks used)
                                    (8, 512, 4096 + 128), (5, 130, 384), (32, 256, 2048 + 128), (16, 100, 1408), (40, 64, 640),
-                                   (8, 512, 4096 + 64), (5, 130, 320), (32, 256, 2048 + 192), (16, 100, 1216)])
+                                   (8, 512, 4096 + 64), (5, 130, 320), (32, 256, 2048 + 192), (16, 100, 1216),
+                                   (8, 512, 4096 + 16), (5, 130, 272), (32, 256, 2048 + 240), (16, 100, 1200), (3, 64, 368)])
 def test_lds_ring_engine(sg, oracle, cfg, shape):
     """The direct-to-LDS ring engine (global_load_lds DMA, conflict-free MFMA reads)."""
     split_k, waves, row_tiles, depth, nt = cfg
@@ -162,7 +163,7 @@ def test_lds_ring_engine(sg, oracle, cfg, shape):
 
 @pytest.mark.parametrize("cfg", [(1, 1, 8), (1, 2, 4), (2, 1, 4), (1, 4, 2), (3, 2, 3), (1, 1, 6)])
 @pytest.mark.parametrize("shape", [(8, 6144, 4096), (5, 130, 512), (16, 1000, 1024), (8, 50, 256), (1, 24, 768), (13, 6144, 1024),
-                                   (32, 96, 512), (8, 6144, 4224), (13, 100, 640), (9, 200, 1344), (16, 72, 448)])
+                                   (32, 96, 512), (8, 6144, 4224), (13, 100, 640), (9, 200, 1344), (16, 72, 448), (8, 120, 1072), (5, 48, 496)])
 def test_lds_ring_24_row_tiles(sg, oracle, cfg, shape):
     """24-row tiles: two 16-row fragments of which the second carries 8 weight rows; its other 8 rows are never fetched
     and never stored (they belong to the next tile).  n a multiple of 24, ragged n (last tile of 10, of 16, of 2 rows),
@@ -781,11 +782,13 @@ def test_decode_sweep_shapes(sg, oracle, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(8, 8192, 29568), (32, 8192, 29568), (1, 2048, 1408), (16, 7168, 1408), (4, 4096, 384),
                                    (24, 1024, 14464), (8, 6144, 4224), (12, 6144, 4224), (32, 512, 28672 + 128),
-                                   (8, 5120, 10944), (32, 5120, 10944), (3, 2048, 320), (16, 6144, 4160), (20, 1024, 14400)])
+                                   (8, 5120, 10944), (32, 5120, 10944), (3, 2048, 320), (16, 6144, 4160), (20, 1024, 14400),
+                                   (8, 4096, 3696), (32, 2048, 7392), (1, 1024, 272), (13, 6144, 4112), (24, 512, 8432)])
 def test_k_with_part_of_a_block_at_its_end(sg, oracle, m, n, k):
-    """k = 256 j + 64, 128 or 192 (the intermediate sizes 29568, 1408 and 10944 of some models): the library's own choice
-    is the per-tile LDS ring, K splits and 24-row tiles included, with the last block loaded from k - 256 and its new
-    64-byte chunks used; against the oracle, and through the row/column-scaled entry point."""
+    """k beyond 256 that is not a multiple of it (the intermediate sizes 29568, 1408 and 10944 of some models, their
+    tensor-parallel shards 3696 and 7392): the library's own choice is the per-tile LDS ring, K splits and 24-row tiles
+    included, with the last block loaded from k - 256 and its new bytes used; against the oracle, and through the
+    row/column-scaled entry point."""
     t, from_table = sg.skinny_gemm_choice(m, n, k)
     assert not from_table and t.engine == 2 and t.persistent_wgs_per_cu == 0
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=3)
@@ -800,7 +803,10 @@ def test_k_with_part_of_a_block_at_its_end(sg, oracle, m, n, k):
     assert oracle.max_rel_err_bf16(bits(D), rowcol_reference(oracle, a8, b8, scale, rs, cs)) <= GEMM_TOL
     # a one-hot activation row picks single weight columns: the columns of the last window must count exactly once
     onehot = np.zeros((m, k), dtype=np.uint8)
-    cols = [k - 1, k - 64, k - 65, k - 128, k - 129, k - 192, k - 193, k - 256, k - 257, 0]
+    tail = k % 256
+    cols = [k - 1, k - 16, k - 17, k - tail, k - tail - 1, k - tail + 15, k - tail + 16, k - 64, k - 65, k - 128, k - 129, k - 192,
+            k - 193, k - 256, k - 257, 0]
+    cols = [c for c in cols if 0 <= c < k]
     for i in range(m):
         onehot[i, cols[i % len(cols)]] = 0x38          # 1.0 in E4M3
     D1 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")

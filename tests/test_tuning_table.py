@@ -133,11 +133,15 @@ def test_search_space_respects_the_fit_rules():
         choice, _ = sg.skinny_gemm_choice(m, n, k)
         assert autotune_fields(choice) in autotune.search_space(m, n, k), (m, n, k, autotune_fields(choice))
     # every k the library takes has candidates, down to a single partial 64-byte stage
-    for k in (16, 32, 48, 80, 4096 + 16):
+    for k in (16, 32, 48, 80, 240):
         space = autotune.search_space(8, 512, k)
         assert space and all(r["engine"] == autotune.ENGINE_DIRECT and r["k_chunks"] == 1 for r in space), k
-    # a k the LDS ring cannot take (not a multiple of 256) gets direct-engine candidates only
-    assert {r["engine"] for r in autotune.search_space(8, 4096, 4096 + 32)} == {autotune.ENGINE_DIRECT}
+    # ... and beyond 256 the per-tile LDS ring next to them, whatever multiple of 16 k is
+    space = autotune.search_space(8, 512, 4096 + 16)
+    assert {r["engine"] for r in space} == {autotune.ENGINE_DIRECT, autotune.ENGINE_LDS}
+    assert all(r["persistent_wgs_per_cu"] == 0 and r["wave_tiles"] & 7 == 0 for r in space if r["engine"] == autotune.ENGINE_LDS)
+    # a k the LDS ring cannot take (below 256 and not a multiple of it) gets direct-engine candidates only
+    assert {r["engine"] for r in autotune.search_space(8, 4096, 240)} == {autotune.ENGINE_DIRECT}
     # mid-batch: the ring must fit 160 KB; 256 x 256 tiles only with a shallow activation ring
     space = autotune.search_space(256, 57344, 8192)
     mid = [r for r in space if r["engine"] == autotune.ENGINE_MID]
@@ -214,7 +218,7 @@ def test_the_heuristics_only_choose_what_the_launchers_take():
     ms = [1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 256, 300, 512]
     ns = [2, 16, 18, 256, 1000, 4096, 4112, 6144, 8192, 10240, 14336, 28672, 57344, 128256]
     ks = [256, 512, 768, 1024, 1536, 2048, 2560, 2816, 3072, 3584, 4096, 5120, 6144, 7168, 8192, 10240, 12288, 14336, 28672,
-          384, 1408, 4224, 14464, 29568, 320, 1344, 10944]    # (the last eight: part of a 256-byte block at the end of K)
+          384, 1408, 4224, 14464, 29568, 320, 1344, 10944, 272, 3696, 7392]    # (from 384 on: part of a 256-byte block at the end of K)
     checked = {1: 0, 2: 0, 4: 0}
     for m in ms:
         for n in ns:
@@ -234,12 +238,13 @@ def test_the_heuristics_only_choose_what_the_launchers_take():
     assert checked[2] > 1000 and checked[4] > 1000, checked
     # k the LDS engines cannot take goes to the direct engine, for every m
     for m in (1, 8, 32, 64):
-        for k in (16, 48, 4096 + 32, 256 + 16) + ((128, 192) if m <= 32 else ()):
+        for k in (16, 48, 240) + ((128, 192) if m <= 32 else (4096 + 32, 256 + 16)):
             choice, _ = sg.skinny_gemm_choice(m, 4096, k)
             assert choice.engine == autotune.ENGINE_DIRECT, (m, k)
     # half a block at the end of K: the per-tile ring up to two 16-row tiles per CU and 32 rows, beyond that the
     # direct engine (the persistent kernels take whole blocks only)
     for m, n, k, engine in ((8, 8192, 29568, 2), (32, 8192, 29568, 2), (1, 2048, 1408, 2), (16, 4096, 384, 2),
-                            (8, 5120, 10944, 2), (24, 2048, 320, 2), (8, 28672, 4224, 1), (32, 8192 + 16, 1408, 1)):
+                            (8, 5120, 10944, 2), (24, 2048, 320, 2), (8, 8192, 3696, 2), (32, 4096, 272, 2),
+                            (8, 28672, 4224, 1), (32, 8192 + 16, 1408, 1)):
         choice, _ = sg.skinny_gemm_choice(m, n, k)
         assert choice.engine == engine and (engine != 2 or (choice.persistent_wgs_per_cu == 0 and choice.wave_tiles & 7 == 0)), (m, n, k)
