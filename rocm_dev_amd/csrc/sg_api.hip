@@ -679,9 +679,9 @@ static Config pick_config(int m, int n, int k, int cu_count) {
     c.persist = 0;
     c.wavetile = 0;
     const int tiles16 = (n + 15) / 16;
-    // (a K with half a block at its end only where the per-tile ring runs, up to two tiles per CU: against the
-    // register-streaming engine, us: 8 x 8192 x 29568 58.1 -> 37, 32 x 8192 x 29568 87.9 -> 45, 8 x 2048 x 1408 4.2 -> 3.2)
-    if (k % 256 == 0 || (lds_half_block_k(k) && m <= 32 && tiles16 <= 2 * cu_count)) {
+    // (a K that is not a multiple of 256 on the per-tile ring: against the register-streaming engine, us:
+    // 8 x 8192 x 29568 58.1 -> 37, 32 x 8192 x 29568 87.9 -> 45, 8 x 2048 x 1408 4.2 -> 3.2)
+    if (k % 256 == 0 || (lds_half_block_k(k) && m <= 32)) {
         c.engine = ENGINE_LDS;
         c.ku = 4;
         const int blocks = (k + 255) / 256;
@@ -696,6 +696,25 @@ static Config pick_config(int m, int n, int k, int cu_count) {
             const int per_split = c.mt == 2 ? 8 : 14;
             few_tiles_split = std::min(std::min(cu_count / tiles16, blocks / per_split), 4);
             if (few_tiles_split < 2) few_tiles_split = 1;
+        }
+        if (tiles16 > 2 * cu_count && k % 256 != 0) {
+            // many tiles and a K the persistent kernels do not take: still one workgroup per tile.  Against the
+            // register-streaming engine, us: 8 x 28672 x 4224 33.3 -> 23.5, 8 x 151936 x 896 33.5 -> 29.5, 8 x 14336 x 4112
+            // 21.9 -> 14.7, 8 x 57344 x 8320 108 -> 79, 16 x 28672 x 2176 19.8 -> 15.0; 32 x 28672 x 4224 45.8 -> 27.1,
+            // 32 x 151936 x 1152 54.9 -> 56.0
+            c.rg = 1;
+            c.waves = 1;
+            c.depth = 4;
+            if (c.mt == 2) {
+                if (blocks >= 8) {
+                    c.rg = 4;
+                    c.waves = 2;
+                    c.depth = 2;
+                } else {
+                    c.rg = 2;
+                }
+            }
+            return c;
         }
         if (tiles16 > 2 * cu_count) {
             // more than two tiles per CU (at exactly two, one-wave workgroups are still 2-3 % ahead up to 16 rows;

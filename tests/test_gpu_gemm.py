@@ -783,7 +783,8 @@ def test_decode_sweep_shapes(sg, oracle, m, n, k):
 @pytest.mark.parametrize("m,n,k", [(8, 8192, 29568), (32, 8192, 29568), (1, 2048, 1408), (16, 7168, 1408), (4, 4096, 384),
                                    (24, 1024, 14464), (8, 6144, 4224), (12, 6144, 4224), (32, 512, 28672 + 128),
                                    (8, 5120, 10944), (32, 5120, 10944), (3, 2048, 320), (16, 6144, 4160), (20, 1024, 14400),
-                                   (8, 4096, 3696), (32, 2048, 7392), (1, 1024, 272), (13, 6144, 4112), (24, 512, 8432)])
+                                   (8, 4096, 3696), (32, 2048, 7392), (1, 1024, 272), (13, 6144, 4112), (24, 512, 8432),
+                                   (8, 28672, 4224), (32, 28672, 4224), (16, 9728, 896), (32, 16384 + 40, 1152)])
 def test_k_with_part_of_a_block_at_its_end(sg, oracle, m, n, k):
     """k beyond 256 that is not a multiple of it (the intermediate sizes 29568, 1408 and 10944 of some models, their
     tensor-parallel shards 3696 and 7392): the library's own choice is the per-tile LDS ring, K splits and 24-row tiles

@@ -241,10 +241,10 @@ def test_the_heuristics_only_choose_what_the_launchers_take():
         for k in (16, 48, 240) + ((128, 192) if m <= 32 else (4096 + 32, 256 + 16)):
             choice, _ = sg.skinny_gemm_choice(m, 4096, k)
             assert choice.engine == autotune.ENGINE_DIRECT, (m, k)
-    # half a block at the end of K: the per-tile ring up to two 16-row tiles per CU and 32 rows, beyond that the
-    # direct engine (the persistent kernels take whole blocks only)
+    # part of a block at the end of K: the per-tile ring up to 32 rows, also on many tiles (the persistent kernels take
+    # whole blocks only)
     for m, n, k, engine in ((8, 8192, 29568, 2), (32, 8192, 29568, 2), (1, 2048, 1408, 2), (16, 4096, 384, 2),
                             (8, 5120, 10944, 2), (24, 2048, 320, 2), (8, 8192, 3696, 2), (32, 4096, 272, 2),
-                            (8, 28672, 4224, 1), (32, 8192 + 16, 1408, 1)):
+                            (8, 28672, 4224, 2), (32, 8192 + 16, 1408, 2), (8, 151936, 896, 2), (40, 4096, 4112, 1)):
         choice, _ = sg.skinny_gemm_choice(m, n, k)
         assert choice.engine == engine and (engine != 2 or (choice.persistent_wgs_per_cu == 0 and choice.wave_tiles & 7 == 0)), (m, n, k)
