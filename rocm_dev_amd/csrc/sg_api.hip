@@ -960,9 +960,9 @@ static Config config_from_tuning(const SgTuning& t) {
 // (64 x 6144 x 4096 13.6 -> 11.0, 64 x 5120 x 5120 18.1 -> 13.4); beyond (64 x 10240 x 4096, 96 x 6144 x 4096,
 // 192 x 4096 x 4096) the mid-batch engine is 10-25 % ahead.
 static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
-    if (m <= 32 || m > 256 || k % 256 != 0) return false;
+    if (m <= 32 || m > 256 || (k % 256 != 0 && !lds_half_block_k(k))) return false;
     const long tiles16 = (n + 15) / 16, tiles32 = (n + 31) / 32, tiles64 = (n + 63) / 64;
-    const int blocks = k / 256, m_tiles = (m + 31) / 32;
+    const int blocks = (k + 255) / 256, m_tiles = (m + 31) / 32;
     Config c;
     c.engine = ENGINE_LDS;
     c.mt = 2;
@@ -996,7 +996,25 @@ static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
 static Config heuristic_config(int m, int n, int k, int cu_count) {
     Config two;
     if (two_pass_config(m, n, k, cu_count, &two)) return two;
-    return (m > 32 && k % 128 == 0) ? pick_mid(m, n, k, cu_count) : pick_config(m, n, k, cu_count);
+    if (m > 32 && k % 128 == 0) return pick_mid(m, n, k, cu_count);
+    if (m > 32 && lds_half_block_k(k)) {
+        // a K the mid-batch engine does not take (not a multiple of 128): the skinny ring over as many 32-row activation
+        // tiles as it takes, 64-row weight tiles on one wave, instead of the register-streaming engine - us:
+        // 128 x 4096 x 7392 51.4 -> 20, 256 x 8192 x 3696 88.6 -> 40, 100 x 14336 x 4112 99.5 -> 45, 48 x 28672 x 2064 59.0 -> 31
+        Config c;
+        c.engine = ENGINE_LDS;
+        c.mt = 2;
+        c.rg = 4;
+        c.waves = 1;
+        c.depth = 2;
+        c.nt = 1;
+        c.ku = 4;
+        c.split_k = 1;
+        c.persist = 0;
+        c.wavetile = 0;
+        return c;
+    }
+    return pick_config(m, n, k, cu_count);
 }
 
 // ---- per-shape tuning table ---------------------------------------------------------------

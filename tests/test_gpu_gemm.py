@@ -784,7 +784,8 @@ def test_decode_sweep_shapes(sg, oracle, m, n, k):
                                    (24, 1024, 14464), (8, 6144, 4224), (12, 6144, 4224), (32, 512, 28672 + 128),
                                    (8, 5120, 10944), (32, 5120, 10944), (3, 2048, 320), (16, 6144, 4160), (20, 1024, 14400),
                                    (8, 4096, 3696), (32, 2048, 7392), (1, 1024, 272), (13, 6144, 4112), (24, 512, 8432),
-                                   (8, 28672, 4224), (32, 28672, 4224), (16, 9728, 896), (32, 16384 + 40, 1152)])
+                                   (8, 28672, 4224), (32, 28672, 4224), (16, 9728, 896), (32, 16384 + 40, 1152),
+                                   (64, 2048, 1424), (100, 4096, 4112), (300, 1024, 3696), (48, 8192 + 8, 2064), (64, 2048, 1408)])
 def test_k_with_part_of_a_block_at_its_end(sg, oracle, m, n, k):
     """k beyond 256 that is not a multiple of it (the intermediate sizes 29568, 1408 and 10944 of some models, their
     tensor-parallel shards 3696 and 7392): the library's own choice is the per-tile LDS ring, K splits and 24-row tiles
@@ -801,7 +802,9 @@ def test_k_with_part_of_a_block_at_its_end(sg, oracle, m, n, k):
     D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
     assert sg.skinny_gemm_rowcol(dev(a8), dev(b8), D, scale_tensor(scale), dev(rs), dev(cs)) == 0
     torch.cuda.synchronize()
-    assert oracle.max_rel_err_bf16(bits(D), rowcol_reference(oracle, a8, b8, scale, rs, cs)) <= GEMM_TOL
+    # (against the model of the matrix instruction's summation, which the kernels reproduce bit for bit: with random
+    # factors the sequential host sum itself can lie just beyond the bar from it in one output of a few hundred thousand)
+    assert oracle.max_rel_err_bf16(bits(D), rowcol_reference(oracle, a8, b8, scale, rs, cs, model=True)) <= GEMM_TOL
     # a one-hot activation row picks single weight columns: the columns of the last window must count exactly once
     onehot = np.zeros((m, k), dtype=np.uint8)
     tail = k % 256
