@@ -136,8 +136,8 @@ typedef struct SgTuning {
     int m_blocks;      /* 16-row activation blocks per tile: 1 (m <= 16 per tile) or 2; mid-batch: 2, 4 or 8 per wavefront */
     int depth;         /* stages in flight per wavefront (register ring / LDS ring slots) */
     int k_chunks;      /* direct engine: 64-byte K chunks per stage (1, 2, 4, 8); LDS ring: fixed 256-byte stage (k a
-                          multiple of 256; one workgroup per tile also takes any other k > 256: the last stage is loaded
-                          from k - 256 and its new bytes used);
+                          multiple of 256; one workgroup per tile and wave_tiles = 1 also take any other k > 256: the last
+                          stage is loaded from k - 256 and its new bytes used);
                           mid-batch: ring slots of the activations, 2 <= k_chunks < depth (anything else = depth) */
     int non_temporal;  /* LDS ring: stream weights with the non-temporal hint */
     int persistent_wgs_per_cu; /* LDS ring: 0 = one workgroup per tile; n > 0 = n persistent workgroups per CU */

@@ -55,9 +55,9 @@ def lds_ring_fits(m, k, r):
     """The LDS-ring kernels' resource rules for one record: ring + resident activations + reduction
     scratch within LDS, and no more DMA instructions in flight than a wave can count."""
     xu = _activation_instructions(m, r["m_blocks"])
-    if k % 256 and not (k % 16 == 0 and k > 256 and not r["persistent_wgs_per_cu"] and not r["wave_tiles"] & 7):
-        return False              # part of a block at the end of K: only the kernel with one workgroup per tile
-    blocks = k // 256
+    if k % 256 and not (k % 16 == 0 and k > 256 and ((not r["persistent_wgs_per_cu"] and not r["wave_tiles"] & 7) or r["wave_tiles"] == 1)):
+        return False              # part of a block at the end of K: one workgroup per tile, or whole tiles per wave
+    blocks = -(-k // 256)
     if r["wave_tiles"] & 8:     # 24-row tiles: two fragments, six weight instructions per stage, one workgroup per tile
         if r["wave_tiles"] != 8 or r["row_tiles"] != 2 or r["m_blocks"] != 1 or r["persistent_wgs_per_cu"]:
             return False

@@ -264,13 +264,13 @@ static unsigned level_persistent_grid(unsigned tiles, size_t most) {
     return (unsigned)((tiles + rounds - 1) / rounds);
 }
 
-// Any k beyond 256 (a multiple of 16, like every k the library takes) also runs on the per-tile ring: the last block
-// is loaded from k - 256 and partly used (the persistent kernels and the kernels that keep the activations resident
-// take multiples of 256 only).
+// Any k beyond 256 (a multiple of 16, like every k the library takes) also runs on the per-tile ring and on the
+// wave-per-tile kernel: the last block is loaded from k - 256 and partly used (the K-split persistent kernels take
+// multiples of 256 only).
 static bool lds_half_block_k(int k) { return k % 256 != 0 && k % 16 == 0 && k > 256; }
 
 static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
-    if (a.k % 256 != 0 && !(lds_half_block_k(a.k) && c.persist == 0 && (c.wavetile & 7) == 0 && !a.A16))
+    if (a.k % 256 != 0 && !(lds_half_block_k(a.k) && !a.A16 && ((c.persist == 0 && (c.wavetile & 7) == 0) || c.wavetile == 1)))
         return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     // wave_tiles bit 3: 24-row tiles (two fragments, the second half used), one workgroup per tile
     const bool rows24 = (c.wavetile & 8) != 0;
@@ -293,7 +293,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         // whole activation matrix resident: one tile row of activations only, no K split
         if (c.split_k != 1 || a.m_tiles != 1 || c.persist < 1) return SG_INVALID_CONFIG;
         mode = 2;
-        lds = (size_t)(a.k / 256) * xu * 1024 + (size_t)c.waves * c.depth * c.rg * 4096 + 4096;
+        lds = (size_t)((a.k + 255) / 256) * xu * 1024 + (size_t)c.waves * c.depth * c.rg * 4096 + 4096;
         DeviceInfo* dev;
         if (int rc = get_device_info(&dev)) return rc;
         size_t want = (size_t)dev->cu_count * c.persist;
@@ -713,6 +713,18 @@ static Config pick_config(int m, int n, int k, int cu_count) {
                 } else {
                     c.rg = 2;
                 }
+            }
+            // ... or, where the whole activation matrix fits LDS beside the rings, whole tiles per wave on a persistent
+            // workgroup per CU (the kernel of the short-K rule below, which takes any k); up to four tiles per CU only
+            // at 17..32 rows, as there
+            const bool fits8 = (size_t)blocks * xu0 * 1024 + 8 * 2 * 4096 + 4096 <= 159 * 1024;
+            const bool fits4 = (size_t)blocks * xu0 * 1024 + 4 * 4 * 4096 + 4096 <= 159 * 1024;
+            if (tiles16 > 4 * cu_count ? fits8 : (c.mt == 2 && fits4)) {
+                c.rg = 1;
+                c.persist = 1;
+                c.wavetile = 1;
+                c.waves = tiles16 > 4 * cu_count ? 8 : 4;
+                c.depth = tiles16 > 4 * cu_count ? 2 : 4;
             }
             return c;
         }

@@ -17,7 +17,8 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
     if constexpr (MODE == 4) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true, true>;
     else if constexpr (MODE == 5) kernel = (a.k & 255) ? lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true, true>
                                                         : lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
-    else if constexpr (MODE == 2) kernel = lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
+    else if constexpr (MODE == 2) kernel = (a.k & 255) ? lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>
+                                                        : lds_gemm_wavetile_kernel<SG_MT, SG_RG, XU, DEPTH, NT>;
     else if constexpr (MODE == 3) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, true>;
     else if constexpr (MODE == 1) kernel = lds_gemm_persistent_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false>;
     else kernel = (a.k & 255) ? lds_gemm_kernel<SG_MT, SG_RG, XU, DEPTH, NT, false, true>   // half a block at the end of K

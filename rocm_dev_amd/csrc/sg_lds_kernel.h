@@ -700,7 +700,9 @@ lds_gemm_persistent_kernel(const StreamArgs a) {
 // waves, which removes a third of the DMA instructions and of the L2 traffic at m = 8.  Wave
 // (workgroup b, wave w) walks tiles b + G*w, + total waves, ...; its weight ring runs across
 // tile boundaries.
-template <int MT, int RG, int XU, int DEPTH, bool NT>
+// TAIL: k not a multiple of 256 - K block `blocks - 1` of both operands is loaded from k - 256 and only its new bytes
+// multiplied (mma_block_tail), as in lds_gemm_kernel.
+template <int MT, int RG, int XU, int DEPTH, bool NT, bool TAIL = false>
 __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_wavetile_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // X[blocks][XU KB] | [wave][DEPTH][RG*4 KB]
 
@@ -715,7 +717,8 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     const int waves = a.waves;
     const int r = lane & 15, g = lane >> 4;
 
-    const int blocks = a.k >> 8;
+    const int blocks = (a.k + 255) >> 8;
+    const size_t tail_shift = TAIL ? (size_t)(256 - (a.k & 255)) : 0;   // how far the last block's window starts early
     const int total_tiles = a.n_tiles * a.m_tiles;
     // tiles are dealt to workgroups first (wave w of workgroup b owns tiles b + G*w, b + G*(w + W), ...), so that a
     // few tiles per CU still put a stream on every CU
@@ -747,7 +750,8 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
         for (int u = 0; u < XU; u++) {
             int row = 4 * u + src_row;
             row = row < a.m ? row : a.m - 1;
-            dma_1kb(a.A + (size_t)row * a.k + ((size_t)kb << 8) + src_col + ((p + (u & 3)) & 3) * 16,
+            dma_1kb(a.A + (size_t)row * a.k + ((size_t)kb << 8) - ((TAIL && kb == blocks - 1) ? tail_shift : 0) + src_col +
+                        ((p + (u & 3)) & 3) * 16,
                     x_lds + (unsigned)(kb * XU + u) * 1024);
         }
         x_issued += XU;
@@ -759,7 +763,7 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
         kb = kb >= blocks ? kb - blocks : kb;
         const int n0 = ((first + j * total_waves) % a.n_tiles) * (16 * RG);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
-        const size_t koff = ((size_t)kb << 8) + src_col;
+        const size_t koff = ((size_t)kb << 8) - ((TAIL && kb == blocks - 1) ? tail_shift : 0) + src_col;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++)
 #pragma unroll
@@ -782,7 +786,8 @@ __global__ void __launch_bounds__(lds_persistent_launch_bound(MT, RG)) lds_gemm_
     auto consume = [&](int i) __attribute__((always_inline)) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES + rd_off;
         const int kb = kb_cur + k_rot >= blocks ? kb_cur + k_rot - blocks : kb_cur + k_rot;   // the K block it holds
-        mma_block_256<MT, RG>(slot, ring + (size_t)kb * (XU * 1024) + rd_off, acc);
+        if (TAIL && kb == blocks - 1) mma_block_tail<MT, RG>(slot, ring + (size_t)kb * (XU * 1024) + rd_off, acc, (int)tail_shift, g);
+        else mma_block_256<MT, RG>(slot, ring + (size_t)kb * (XU * 1024) + rd_off, acc);
     };
 
     const float scale = a.scale ? a.scale[0] : 1.0f;

@@ -28,7 +28,7 @@ def expect_lds(m, n, k, r):
     persist, wt = r["persistent_wgs_per_cu"], r["wave_tiles"]
     if k % 256:
         # part of a block at the end of K: only the kernel with one workgroup per tile (16-, 32-, 64- or 24-row tiles)
-        if not (k % 16 == 0 and k > 256 and persist == 0 and wt & 7 == 0):
+        if not (k % 16 == 0 and k > 256 and ((persist == 0 and wt & 7 == 0) or wt == 1)):
             return 3
     blocks = k // 256
     if not (1 <= waves <= 16 and depth >= 1 and rg >= 1 and mt in (1, 2) and 1 <= sk <= blocks):
@@ -51,7 +51,7 @@ def expect_lds(m, n, k, r):
     if wt == 1:                                           # every wave owns whole tiles, activations resident in LDS
         if sk != 1 or m_tiles != 1 or persist < 1:
             return INVALID
-        lds = blocks * xu * 1024 + waves * depth * rg * 4096 + 4096
+        lds = -(-k // 256) * xu * 1024 + waves * depth * rg * 4096 + 4096
         if lds > LDS_USABLE:
             return INVALID
         if waves * 64 > 1024:

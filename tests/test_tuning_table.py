@@ -139,7 +139,8 @@ def test_search_space_respects_the_fit_rules():
     # ... and beyond 256 the per-tile LDS ring next to them, whatever multiple of 16 k is
     space = autotune.search_space(8, 512, 4096 + 16)
     assert {r["engine"] for r in space} == {autotune.ENGINE_DIRECT, autotune.ENGINE_LDS}
-    assert all(r["persistent_wgs_per_cu"] == 0 and r["wave_tiles"] & 7 == 0 for r in space if r["engine"] == autotune.ENGINE_LDS)
+    assert all((r["persistent_wgs_per_cu"] == 0 and r["wave_tiles"] & 7 == 0) or r["wave_tiles"] == 1
+               for r in space if r["engine"] == autotune.ENGINE_LDS)
     # a k the LDS ring cannot take (below 256 and not a multiple of it) gets direct-engine candidates only
     assert {r["engine"] for r in autotune.search_space(8, 4096, 240)} == {autotune.ENGINE_DIRECT}
     # mid-batch: the ring must fit 160 KB; 256 x 256 tiles only with a shallow activation ring
@@ -250,4 +251,5 @@ def test_the_heuristics_only_choose_what_the_launchers_take():
                             (8, 28672, 4224, 2), (32, 8192 + 16, 1408, 2), (8, 151936, 896, 2), (40, 4096, 4112, 2), (300, 8192, 3696, 2),
                             (64, 2048, 1408, 2), (300, 8192, 1408, 4), (64, 4096, 240, 1)):
         choice, _ = sg.skinny_gemm_choice(m, n, k)
-        assert choice.engine == engine and (engine != 2 or (choice.persistent_wgs_per_cu == 0 and choice.wave_tiles & 7 == 0)), (m, n, k)
+        assert choice.engine == engine and (engine != 2 or choice.wave_tiles == 1 or
+                                            (choice.persistent_wgs_per_cu == 0 and choice.wave_tiles & 7 == 0)), (m, n, k)
