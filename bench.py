@@ -72,6 +72,10 @@ def main():
                          "on cold weights through the library's choice and three times through the one-wave-workgroup kernel "
                          "it replaced, after three 256 MiB copies of known traffic, and exit (for L2 / HBM traffic counter runs; "
                          "prints no JSON line)")
+    ap.add_argument("--k-tail-counters", action="store_true",
+                    help="K that 256 does not divide: launch the library's choice (LDS ring with a partly used last stage) and the "
+                         "register-streaming engine it replaced three times each on cold weights, next to the neighbouring "
+                         "multiple of 256, and exit (for kernel traces and HBM-traffic counters)")
     ap.add_argument("--n-sweep", action="store_true",
                     help="only run 8 x N x 4096 for N = 4096 ... 57344 (1 ... 14 sixteen-row tiles per CU): the library's own "
                          "choice, the per-tile kernel (one wave, eight slots) and the read-only streaming yardstick "
@@ -419,6 +423,37 @@ def main():
                 if rc != 0:
                     raise RuntimeError("sg_sparse24_gemm: %s" % sg.strerror(rc))
             torch.cuda.synchronize()
+        return
+
+    if args.k_tail_counters:
+        import ctypes
+        one = torch.ones(1, device="cuda")
+        for (m, n, k, k256) in ((8, 8192, 29568, 29696), (32, 8192, 29568, 29696), (8, 151936, 896, 1024), (8, 28672, 4224, 4096),
+                                (8, 2048, 1408, 1536), (8, 8192, 3696, 3840), (128, 4096, 7392, 7424)):
+            for kk in (k, k256):
+                copies = max(3, int(COLD_BYTES // (n * kk)) + 1)
+                wb = [torch.randint(0, 0x7E, (n, kk), device="cuda", dtype=torch.uint8) for _ in range(min(copies, 6))]
+                a8 = torch.randint(0, 0x7E, (m, kk), device="cuda", dtype=torch.uint8)
+                d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+                for i in range(3):
+                    rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % len(wb)].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, kk, kk, None)
+                    if rc != 0:
+                        raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
+                torch.cuda.synchronize()
+                if kk == k:
+                    # the register-streaming engine as it was chosen for such k: 64- or 128-byte stages, four or eight
+                    # waves sharing K, two 16-row tiles per wave on very wide matrices
+                    ku = 2 if k % 128 == 0 else 1
+                    stages = -(-k // (64 * ku))
+                    waves = 8 if stages >= 16 else 4
+                    rec = sg.SgTuning(1, 1, waves, 2 if n >= 8 * 16 * 256 else 1, 1 if m <= 16 else 2, 4 if ku == 1 else 2, ku, 1, 0, 0)
+                    for i in range(3):
+                        rc = lib.sg_skinny_gemm_tuned(a8.data_ptr(), wb[i % len(wb)].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k,
+                                                      ctypes.byref(rec), None)
+                        if rc != 0:
+                            raise RuntimeError("sg_skinny_gemm_tuned (direct): %s" % sg.strerror(rc))
+                    torch.cuda.synchronize()
+                del wb
         return
 
     if args.mid_batch_counters:
