@@ -984,6 +984,25 @@ static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
     c.persist = 0;
     c.wavetile = 0;
     c.depth = 2;
+    if (blocks >= 64) {
+        // K of 16384 or more: two K splits on the tile that still fits the round with them, or the mid-batch engine
+        // (which splits up to four ways).  us: 40 x 1024 x 28672 20.9 unsplit -> 14.3 (mid-batch 24.6), 128 x 1024 x 28672
+        // 23.7 -> 18.8 (26.5), 64 x 2048 x 28672 25.7 -> 21.2 (28.2), 64 x 2048 x 20480 19.7 -> 16.9 (23.5); 48 x 3072 x 28672
+        // and 64 x 4096 x 28672, where only the unsplit ring fits, 34.9 and 36.1 against 28.5 and 31.7 for the mid-batch engine
+        c.split_k = 2;
+        if (tiles16 * m_tiles * 2 <= cu_count) {
+            c.rg = 1;
+            c.waves = 2;
+            c.depth = 3;
+        } else if (tiles32 * m_tiles * 2 <= cu_count) {
+            c.rg = 2;
+            c.waves = 3;
+        } else {
+            return false;
+        }
+        *out = c;
+        return true;
+    }
     if (tiles16 * m_tiles <= cu_count) {           // 16-row tiles: every (tile, activation tile) pair gets a CU
         c.rg = 1;
         c.waves = 2;

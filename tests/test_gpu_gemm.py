@@ -553,6 +553,18 @@ def test_lds_ring_wave_tiles(sg, oracle, cfg, shape):
     assert np.array_equal(bits(D2), got)
 
 
+@pytest.mark.parametrize("m,n,k,tile_rows", [(40, 1024, 28672, 16), (64, 2048, 20480, 32), (128, 1024, 16384, 32)])
+def test_several_activation_tiles_and_a_very_long_k(sg, oracle, m, n, k, tile_rows):
+    """From K = 16384 on the skinny ring over several activation tiles splits K in two where the round still holds both
+    splits of every (weight tile, activation tile) pair; against the oracle."""
+    t, from_table = sg.skinny_gemm_choice(m, n, k)
+    assert not from_table and (t.engine, t.m_blocks, 16 * t.row_tiles, t.split_k) == (2, 2, tile_rows, 2)
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=13)
+    ref = gemm_reference(oracle, a8, b8, scale)
+    got = _run_fast(sg, a8, b8, scale)
+    assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
+
+
 @pytest.mark.parametrize("field", ["waves", "row_tiles", "m_blocks", "depth", "k_chunks", "split_k"])
 @pytest.mark.parametrize("engine", [1, 2, 4])
 @pytest.mark.parametrize("bad", [0, -1, 1000])
