@@ -121,7 +121,7 @@ def search_space(m, n, k):
     """Candidate records for one shape, already filtered by the fit rules above.  The library stays the
     authority: a candidate it has no kernel for comes back SG_INVALID_CONFIG and is skipped."""
     out = []
-    if m > 32 and k % 128 == 0:
+    if m > 32 and (k % 128 == 0 or (k % 16 == 0 and k > 128)):     # (a partial last block: the library has builds for some)
         for waves, rt, mb, depth, dx, sk in itertools.product((4, 8, 14), (2, 4), (2, 4, 8), (2, 3, 4, 6), (0, 2, 3), (1, 2, 3, 4, 5, 6, 8)):
             if dx and dx >= depth:
                 continue
@@ -133,7 +133,7 @@ def search_space(m, n, k):
             if mid_fits(k, r):
                 out.append(r)
         # the skinny LDS ring over several 32-row activation tiles (what the library runs on small weight matrices)
-        if m <= 256 and k % 256 == 0:
+        if m <= 256 and (k % 256 == 0 or (k % 16 == 0 and k > 256)):
             for sk, waves, rt, depth in itertools.product((1, 2), (1, 2, 3, 4), (1, 2, 4), (2, 3, 4)):
                 r = record(ENGINE_LDS, sk, waves, rt, 2, depth, 4, 1, 0, 0)
                 if lds_ring_fits(m, k, r):

@@ -414,8 +414,12 @@ static int launch_ring(const RingConfig& c, StreamArgs a, hipStream_t stream) {
 
 // Mid-batch engine: c.rg = 16-row weight fragments per wave (2 or 4), c.mt = 16-row activation
 // fragments per wave (2, 4 or 8); a workgroup tile is 16*c.rg*(waves/2) weight rows x 32*c.mt activation rows.
+// The mid-batch kernel's stage is 128 bytes of K; a k beyond 128 that is only a multiple of 16 runs in the builds with a
+// partial last block, which exist for the tiles and rings pick_mid chooses.
+static bool mid_partial_block_k(int k) { return k % 128 != 0 && k % 16 == 0 && k > 128; }
+
 static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) {
-    if (a.k % 128 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (a.k % 128 != 0 && !mid_partial_block_k(a.k)) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if ((c.rg != 2 && c.rg != 4) || (c.mt != 2 && c.mt != 4 && c.mt != 8) || c.depth < 2) return SG_INVALID_CONFIG;
     if (c.waves != 4 && c.waves != 8 && c.waves != 14) return SG_INVALID_CONFIG;
     const int wn = c.waves / 2;                   // waves = wn (along n) x 2 (along m)
@@ -458,7 +462,7 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4}, {256, 128, 8}, {224, 128, 14},
                                  {256, 64, 8}, {224, 64, 14}, {128, 256, 8}, {256, 256, 8}, {224, 256, 14}};
     const int bm_max = m <= 64 ? 64 : (m <= 128 ? 128 : 256);
-    const int blocks = k / 128;
+    const int blocks = (k + 127) / 128;
     Config best;
     long best_rounds = -1, best_wgs = 0;
     const Tile* best_tile = nullptr;
@@ -1027,24 +1031,9 @@ static bool two_pass_config(int m, int n, int k, int cu_count, Config* out) {
 static Config heuristic_config(int m, int n, int k, int cu_count) {
     Config two;
     if (two_pass_config(m, n, k, cu_count, &two)) return two;
-    if (m > 32 && k % 128 == 0) return pick_mid(m, n, k, cu_count);
-    if (m > 32 && lds_half_block_k(k)) {
-        // a K the mid-batch engine does not take (not a multiple of 128): the skinny ring over as many 32-row activation
-        // tiles as it takes, 64-row weight tiles on one wave, instead of the register-streaming engine - us:
-        // 128 x 4096 x 7392 51.4 -> 20, 256 x 8192 x 3696 88.6 -> 40, 100 x 14336 x 4112 99.5 -> 45, 48 x 28672 x 2064 59.0 -> 31
-        Config c;
-        c.engine = ENGINE_LDS;
-        c.mt = 2;
-        c.rg = 4;
-        c.waves = 1;
-        c.depth = 2;
-        c.nt = 1;
-        c.ku = 4;
-        c.split_k = 1;
-        c.persist = 0;
-        c.wavetile = 0;
-        return c;
-    }
+    // (a k that is not a multiple of 128 runs in the mid-batch kernel's builds with a partial last block: against the
+    // skinny ring over 64-row weight tiles, which took such k before, us: 128 x 4096 x 7392 19.9 -> see the design notes)
+    if (m > 32 && (k % 128 == 0 || mid_partial_block_k(k))) return pick_mid(m, n, k, cu_count);
     return pick_config(m, n, k, cu_count);
 }
 

@@ -5,9 +5,9 @@
 
 namespace sg {
 
-template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH>
+template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH, bool TAIL = false>
 static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
-    auto kernel = mid_gemm_kernel<RGW, MH, DEPTH, WN, DX>;
+    auto kernel = mid_gemm_kernel<RGW, MH, DEPTH, WN, DX, TAIL>;
     static LdsGranted granted;
     if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), lds, granted)) return rc;
     kernel<<<dim3(grid), dim3(WN * 128), lds, stream>>>(a);
@@ -35,7 +35,24 @@ static int launch_one(const StreamArgs& a, unsigned grid, size_t lds, hipStream_
     if (rgw == 2 && mh == MH_ && depth == DEPTH_ && dx == DX_ && wn == 7)                      \
         return launch_one<2, MH_, DEPTH_, 7, DX_>(a, grid, lds, stream);
 
+// k not a multiple of 128: the tiles and rings the heuristics choose (pick_mid), built with the partial last block
+#define SG_TAIL(RGW_, MH_, DEPTH_, WN_, DX_)                                                   \
+    if (rgw == RGW_ && mh == MH_ && depth == DEPTH_ && dx == DX_ && wn == WN_)                 \
+        return launch_one<RGW_, MH_, DEPTH_, WN_, DX_, true>(a, grid, lds, stream);
+
+static int launch_mid_tail(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, unsigned grid, size_t lds,
+                           hipStream_t stream) {
+    SG_TAIL(2, 2, 4, 2, 4) SG_TAIL(2, 4, 4, 2, 4)                          // 64 x 64, 64 x 128 on four waves
+    SG_TAIL(2, 2, 4, 4, 4) SG_TAIL(2, 4, 4, 4, 4) SG_TAIL(2, 8, 3, 4, 3)   // 128 x 64, 128 x 128, 128 x 256
+    SG_TAIL(2, 2, 4, 4, 2)                                                 // two 128 x 64 workgroups per CU
+    SG_TAIL(4, 2, 4, 4, 4) SG_TAIL(4, 2, 3, 4, 3) SG_TAIL(4, 4, 3, 4, 3)   // 256 x 64 (unsplit, split), 256 x 128
+    SG_TAIL(4, 8, 3, 4, 2) SG_TAIL(4, 8, 2, 4, 2)                          // 256 x 256 (unsplit, split)
+    SG_TAIL(2, 2, 4, 7, 4) SG_TAIL(2, 4, 4, 7, 3) SG_TAIL(2, 8, 3, 7, 2)   // 224 x 64, 224 x 128, 224 x 256
+    return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+}
+
 int launch_mid(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
+    if (a.k & 127) return launch_mid_tail(rgw, mh, depth, dx, wn, a, grid, lds, stream);
     SG_CASE_7(8, 3, 2) SG_CASE_7(8, 2, 2)                                       // 224 x 256: 84 + 64 KB
     SG_CASE_7(4, 4, 2) SG_CASE_7(4, 4, 3) SG_CASE_7(4, 3, 3) SG_CASE_7(4, 3, 2)  // 224 x 128
     SG_CASE_7(2, 4, 2) SG_CASE_7(2, 4, 4) SG_CASE_7(2, 3, 3)                     // 224 x 64

@@ -50,7 +50,11 @@ constexpr int mid_activation_waves(int instr, int waves) {
     return best;
 }
 
-template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH>
+// TAIL: k is not a multiple of 128 (but of 16, and beyond 128).  The last 128-byte K block of both operands is loaded
+//      from k - 128 - a window that ends with the row, nothing past it is read - and the activation fragments of that
+//      stage are zero in the 16-byte pieces the block before has already multiplied: lane (r, g) holds pieces g and
+//      g + 4 of a row, so that is a per-lane select.  (A build of its own: the loop for whole blocks stays as it is.)
+template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH, bool TAIL = false>
 __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) {
     // [DEPTH][W rows][128] | [DX][X rows][128], then (split-K only) 16 bytes for the arrival broadcast; no
     // static LDS, so that two workgroups of exactly half the CU's LDS can share a CU
@@ -113,8 +117,10 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     const int m0 = tile_m * BM;
 
     int b_begin, b_end;
-    split_range(a, a.k >> 7, split, b_begin, b_end);   // 128-byte K blocks
+    const int blocks_total = (a.k + 127) >> 7;         // 128-byte K blocks, the last of them partial in a TAIL build
+    split_range(a, blocks_total, split, b_begin, b_end);
     const int n_blk = b_end - b_begin;
+    const int old_pieces = TAIL ? (128 - (a.k & 127)) >> 4 : 0;   // 16-byte pieces of the last window that are not new
     // Every workgroup walks its K range from a different starting block (and wraps): workgroups that start
     // together would otherwise ask one L2 for the same activation lines at the same moment, block after
     // block, and queue up at one channel.  The start depends on the weight tile only, so the workgroups that
@@ -147,13 +153,17 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     const unsigned ring_lds = lds_addr(ring);
     // DMA instruction i of a stage's refill: the activation instructions come first, then the weights'
     auto issue_one = [&](int i, int sx, int sw) __attribute__((always_inline)) {
+        // byte offset of K block kb inside a row: the last block of a TAIL build starts early, so that it ends with the row
+        auto k_offset = [&](int kb) __attribute__((always_inline)) {
+            return ((size_t)kb << 7) - ((TAIL && kb == blocks_total - 1) ? (size_t)(old_pieces << 4) : 0);
+        };
         if (i < X_INSTR) {
             if (loads_x && sx < n_blk)
-                dma_1kb(xsrc[i] + ((size_t)k_block(sx) << 7),
+                dma_1kb(xsrc[i] + k_offset(k_block(sx)),
                         ring_lds + DEPTH * W_BYTES + (unsigned)(sx % DX) * X_BYTES + (XW * i + wave) * 1024);
         } else {
             if (sw < n_blk)
-                dma_1kb_stream(wsrc[i - X_INSTR] + ((size_t)k_block(sw) << 7),
+                dma_1kb_stream(wsrc[i - X_INSTR] + k_offset(k_block(sw)),
                                ring_lds + (unsigned)(sw % DEPTH) * W_BYTES + (WAVES * (i - X_INSTR) + wave) * 1024);
         }
     };
@@ -194,6 +204,18 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
             const i32x4 hi = *reinterpret_cast<const i32x4*>(p + rd1);
             return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
         };
+        // TAIL: the stage that holds the last window - its activation pieces below the boundary are zero
+        const bool last_window = TAIL && k_block(s) == blocks_total - 1;
+        const bool zero_lo = last_window && g < old_pieces, zero_hi = last_window && g + 4 < old_pieces;
+        auto read_x_frag = [&](const uint8_t* p) __attribute__((always_inline)) {
+            i32x4 lo = *reinterpret_cast<const i32x4*>(p + rd0);
+            i32x4 hi = *reinterpret_cast<const i32x4*>(p + rd1);
+            if constexpr (TAIL) {
+                if (zero_lo) lo = i32x4{0, 0, 0, 0};
+                if (zero_hi) hi = i32x4{0, 0, 0, 0};
+            }
+            return i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        };
         // the wave's weight fragments stay in registers for the stage; its activation fragments are
         // streamed one ahead of the MFMAs that use them, so that only the first reads of a stage are
         // exposed and the rest of the LDS traffic runs under the matrix cores
@@ -201,10 +223,10 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
 #pragma unroll
         for (int rg = 0; rg < RGW; rg++) w[rg] = read_frag(wslot + rg * 2048);
         i32x8 x[2];
-        x[0] = read_frag(xslot);
+        x[0] = read_x_frag(xslot);
 #pragma unroll
         for (int mb = 0; mb < MH; mb++) {
-            if (mb + 1 < MH) x[(mb + 1) & 1] = read_frag(xslot + (mb + 1) * 2048);
+            if (mb + 1 < MH) x[(mb + 1) & 1] = read_x_frag(xslot + (mb + 1) * 2048);
 #pragma unroll
             for (int i = mb * PER_STAGE / MH; i < (mb + 1) * PER_STAGE / MH; i++) issue_one(i, sx, sw);
             __builtin_amdgcn_sched_barrier(0);
@@ -229,11 +251,17 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         __builtin_amdgcn_sched_barrier(0);
         const uint8_t* wslot = ring + (size_t)(s % DEPTH) * W_BYTES + w_base;
         const uint8_t* xslot = ring + (size_t)DEPTH * W_BYTES + (size_t)(s % DX) * X_BYTES + x_base;
+        const bool last_window = TAIL && k_block(s) == blocks_total - 1;
+        const bool zero_lo = last_window && g < old_pieces, zero_hi = last_window && g + 4 < old_pieces;
         i32x8 x[MH];
 #pragma unroll
         for (int mb = 0; mb < MH; mb++) {
-            const i32x4 lo = *reinterpret_cast<const i32x4*>(xslot + mb * 2048 + rd0);
-            const i32x4 hi = *reinterpret_cast<const i32x4*>(xslot + mb * 2048 + rd1);
+            i32x4 lo = *reinterpret_cast<const i32x4*>(xslot + mb * 2048 + rd0);
+            i32x4 hi = *reinterpret_cast<const i32x4*>(xslot + mb * 2048 + rd1);
+            if constexpr (TAIL) {
+                if (zero_lo) lo = i32x4{0, 0, 0, 0};
+                if (zero_hi) hi = i32x4{0, 0, 0, 0};
+            }
             x[mb] = i32x8{lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
         }
 #pragma unroll

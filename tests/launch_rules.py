@@ -110,13 +110,29 @@ _MID_DX = {(4, 8, 3, 2), (4, 4, 4, 2), (4, 4, 4, 3), (4, 4, 3, 2), (4, 2, 4, 2),
            (2, 8, 6, 2), (2, 4, 6, 2), (2, 4, 6, 3), (2, 4, 4, 2), (2, 2, 6, 2), (2, 2, 6, 3), (2, 2, 4, 2)}
 
 
+# (row_tiles, m_blocks, depth, waves along n, activation slots) built with a partial last K block
+_MID_TAIL = {(2, 2, 4, 2, 4), (2, 4, 4, 2, 4), (2, 2, 4, 4, 4), (2, 4, 4, 4, 4), (2, 8, 3, 4, 3), (2, 2, 4, 4, 2), (4, 2, 4, 4, 4),
+             (4, 2, 3, 4, 3), (4, 4, 3, 4, 3), (4, 8, 3, 4, 2), (4, 8, 2, 4, 2), (2, 2, 4, 7, 4), (2, 4, 4, 7, 3), (2, 8, 3, 7, 2)}
+
+
 def expect_mid(m, n, k, r):
     """Mid-batch engine (SgTuning.engine = 4): a workgroup tile is 16*row_tiles*(waves/2) weight rows by
     32*m_blocks activation rows, `depth` weight slots and `k_chunks` (or depth) activation slots of
     128 bytes of K."""
     waves, rg, mt, depth, sk, dx = r["waves"], r["row_tiles"], r["m_blocks"], r["depth"], r["split_k"], r["k_chunks"]
     if k % 128:
-        return 3
+        # a partial last block: only beyond 128, and only in the builds listed below
+        if k % 16 or k <= 128:
+            return 3
+        if rg not in (2, 4) or mt not in (2, 4, 8) or depth < 2 or waves not in (4, 8, 14):
+            return INVALID
+        if not 1 <= sk <= k // 128:
+            return INVALID
+        d = dx if 2 <= dx < depth else depth
+        wn_ = waves // 2
+        if (depth * 16 * rg * wn_ + d * 32 * mt) * 128 + (16 if sk > 1 else 0) > 160 * 1024:
+            return INVALID
+        return OK if (rg, mt, depth, wn_, d) in _MID_TAIL else 3
     if rg not in (2, 4) or mt not in (2, 4, 8) or depth < 2 or waves not in (4, 8, 14):
         return INVALID
     wn = waves // 2

@@ -456,7 +456,9 @@ MID_CONFIGS = [
 
 @pytest.mark.parametrize("cfg", MID_CONFIGS)
 @pytest.mark.parametrize("shape", [(64, 512, 1024), (40, 130, 2048), (128, 1024, 2048), (256, 640, 4096), (200, 256, 4096),
-                                   (300, 128, 1536), (33, 64, 128)])
+                                   (300, 128, 1536), (33, 64, 128),
+                                   # a partial last 128-byte block (the builds that exist run, the others say so)
+                                   (64, 512, 1040), (128, 1024, 2160), (200, 256, 4208), (40, 130, 272), (300, 128, 1648)])
 def test_mid_batch_engine(sg, oracle, cfg, shape):
     """32 < m: weights streamed once, 2 x 2 or 4 x 2 waves per tile, 16x16x128 scaled MFMA with unit scales."""
     rgw, mh, depth, split_k, waves = cfg[:5]
@@ -800,14 +802,18 @@ def test_decode_sweep_shapes(sg, oracle, m, n, k):
                                    (8, 4096, 3696), (32, 2048, 7392), (1, 1024, 272), (13, 6144, 4112), (24, 512, 8432),
                                    (8, 28672, 4224), (32, 28672, 4224), (16, 9728, 896), (32, 16384 + 40, 1152),
                                    (64, 2048, 1424), (100, 4096, 4112), (300, 1024, 3696), (48, 8192 + 8, 2064), (64, 2048, 1408),
-                                   (8, 151936, 896), (16, 32768, 2192), (32, 24576, 1152), (4, 28672, 4224)])
+                                   (8, 151936, 896), (16, 32768, 2192), (32, 24576, 1152), (4, 28672, 4224),
+                                   # more than 32 rows: the mid-batch engine's builds with a partial last 128-byte block
+                                   (64, 8192, 3696), (128, 4096, 7392), (256, 8192, 1424), (200, 14336, 2064), (64, 28672, 1168),
+                                   (320, 4096, 4112), (448, 28672, 400), (100, 57344, 272), (40, 10240, 10944)])
 def test_k_with_part_of_a_block_at_its_end(sg, oracle, m, n, k):
     """k beyond 256 that is not a multiple of it (the intermediate sizes 29568, 1408 and 10944 of some models, their
     tensor-parallel shards 3696 and 7392): the library's own choice is the per-tile LDS ring, K splits and 24-row tiles
-    included, with the last block loaded from k - 256 and its new bytes used; against the oracle, and through the
-    row/column-scaled entry point."""
+    included, or above 32 rows the mid-batch engine, with the last block loaded from k - 256 (k - 128) and its new bytes
+    used; against the oracle, and through the row/column-scaled entry point."""
     t, from_table = sg.skinny_gemm_choice(m, n, k)
-    assert not from_table and t.engine == 2 and (t.persistent_wgs_per_cu == 0 or t.wave_tiles == 1)
+    assert not from_table and (t.engine == 4 if m > 256 else t.engine in (2, 4) if m > 32 else t.engine == 2)
+    assert t.engine == 4 or t.persistent_wgs_per_cu == 0 or t.wave_tiles == 1
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=3)
     ref = gemm_reference(oracle, a8, b8, scale)
     got = _run_fast(sg, a8, b8, scale)

@@ -230,9 +230,7 @@ def test_the_heuristics_only_choose_what_the_launchers_take():
                 checked[r["engine"]] += 1
                 if r["engine"] == autotune.ENGINE_LDS:
                     # (more than 32 rows on a small matrix run the skinny ring over several activation tiles)
-                    # (... up to 256 rows, or any number of them where k is no multiple of 128 and the mid-batch engine
-                    # does not apply)
-                    assert (m <= 256 or k % 128) and launch_rules.expect_lds(m, n, k, r) == launch_rules.OK, (m, n, k, r)
+                    assert m <= 256 and launch_rules.expect_lds(m, n, k, r) == launch_rules.OK, (m, n, k, r)
                     assert m <= 32 or (r["persistent_wgs_per_cu"] == 0 and r["wave_tiles"] == 0 and r["m_blocks"] == 2), (m, n, k, r)
                 elif r["engine"] == autotune.ENGINE_MID:
                     assert launch_rules.expect_mid(m, n, k, r) == launch_rules.OK, (m, n, k, r)
@@ -241,15 +239,15 @@ def test_the_heuristics_only_choose_what_the_launchers_take():
     assert checked[2] > 1000 and checked[4] > 1000, checked
     # k the LDS engines cannot take goes to the direct engine, for every m
     for m in (1, 8, 32, 64):
-        for k in (16, 48, 240) + ((128, 192) if m <= 32 else ()):
+        for k in (16, 48, 112) + ((128, 192, 240) if m <= 32 else ()):
             choice, _ = sg.skinny_gemm_choice(m, 4096, k)
             assert choice.engine == autotune.ENGINE_DIRECT, (m, k)
-    # part of a block at the end of K: the per-tile ring, also on many tiles (the persistent kernels take whole blocks
-    # only) and, where k is no multiple of 128 either, for more than 32 rows (the mid-batch engine does not apply)
+    # part of a block at the end of K: the per-tile ring, also on many tiles (the K-split persistent kernels take whole
+    # blocks only); above 32 rows the skinny ring over several activation tiles or the mid-batch engine, as for other k
     for m, n, k, engine in ((8, 8192, 29568, 2), (32, 8192, 29568, 2), (1, 2048, 1408, 2), (16, 4096, 384, 2),
                             (8, 5120, 10944, 2), (24, 2048, 320, 2), (8, 8192, 3696, 2), (32, 4096, 272, 2),
-                            (8, 28672, 4224, 2), (32, 8192 + 16, 1408, 2), (8, 151936, 896, 2), (40, 4096, 4112, 2), (300, 8192, 3696, 2),
-                            (64, 2048, 1408, 2), (300, 8192, 1408, 4), (64, 4096, 240, 1)):
+                            (8, 28672, 4224, 2), (32, 8192 + 16, 1408, 2), (8, 151936, 896, 2), (40, 4096, 4112, 2), (300, 8192, 3696, 4),
+                            (64, 2048, 1408, 2), (300, 8192, 1408, 4), (64, 4096, 240, 4), (64, 8192, 10944, 4), (64, 4096, 112, 1)):
         choice, _ = sg.skinny_gemm_choice(m, n, k)
         assert choice.engine == engine and (engine != 2 or choice.wave_tiles == 1 or
                                             (choice.persistent_wgs_per_cu == 0 and choice.wave_tiles & 7 == 0)), (m, n, k)
