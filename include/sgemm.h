@@ -127,7 +127,9 @@ int sg_skinny_gemm_rowcol(const uint8_t* A, const uint8_t* B, void* D_bf16, cons
  * (grid.py:106-116); this is the run-time equivalent a tuning driver sweeps. */
 typedef struct SgTuning {
     int engine;        /* 0 library's choice, 1 direct (global -> VGPR -> MFMA), 2 LDS ring (global -> LDS DMA -> MFMA),
-                          4 mid-batch (32 < m: weights streamed once, both operands staged in LDS for 2x2 or 4x2 waves) */
+                          4 mid-batch (32 < m: weights streamed once, both operands staged in LDS for 2x2 or 4x2 waves;
+                          k a multiple of 128, or - for the tile and ring combinations the library itself chooses - any
+                          multiple of 16 beyond 128, the last 128-byte stage then loaded from k - 128) */
     int split_k;       /* workgroups sharing one output tile along K */
     int waves;         /* wavefronts per workgroup, sharing the tile along K (1..16); mid-batch: 4 (2 along n x 2 along m),
                           8 (4 x 2) or 14 (7 x 2, row_tiles = 2: 224-row tiles), each owning row_tiles x m_blocks
