@@ -32,7 +32,7 @@ COLD_BYTES = 640e6          # per shape: distinct weight bytes cycled through (>
 # HBM bytes per launch of the dominant kernel (gate_up, M = 8), measured off-line with two
 # rocprofv3 --pmc runs (FETCH_SIZE x 1.9998, WRITE_SIZE x 1.0, factors from a 256 MiB copy);
 # the runs and their arithmetic are in profiles/dense_gemm_decode_step_m8_pmc_traffic.md
-RECORDED_TRAFFIC = {"bytes": 118353717, "source": "profiles/dense_gemm_decode_step_m8_pmc_traffic.md",
+RECORDED_TRAFFIC = {"bytes": 118344281, "source": "profiles/dense_gemm_decode_step_m8_pmc_traffic.md",
                     # the kernel configuration the counters were read on; another configuration reports no traffic
                     "tuning": {"engine": 2, "waves": 8, "row_tiles": 1, "depth": 2, "persistent_wgs_per_cu": 1, "wave_tiles": 6}}
 
