@@ -805,7 +805,8 @@ def test_decode_sweep_shapes(sg, oracle, m, n, k):
                                    (8, 151936, 896), (16, 32768, 2192), (32, 24576, 1152), (4, 28672, 4224),
                                    # more than 32 rows: the mid-batch engine's builds with a partial last 128-byte block
                                    (64, 8192, 3696), (128, 4096, 7392), (256, 8192, 1424), (200, 14336, 2064), (64, 28672, 1168),
-                                   (320, 4096, 4112), (448, 28672, 400), (100, 57344, 272), (40, 10240, 10944)])
+                                   (320, 4096, 4112), (448, 28672, 400), (100, 57344, 272), (40, 10240, 10944),
+                                   (64, 512, 144), (100, 300, 240), (33, 64, 160), (300, 8192, 208)])
 def test_k_with_part_of_a_block_at_its_end(sg, oracle, m, n, k):
     """k beyond 256 that is not a multiple of it (the intermediate sizes 29568, 1408 and 10944 of some models, their
     tensor-parallel shards 3696 and 7392): the library's own choice is the per-tile LDS ring, K splits and 24-row tiles
