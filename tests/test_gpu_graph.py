@@ -32,6 +32,12 @@ def test_replays_match_eager(oracle):
     jobs.append(("split-K ring", *gemm(32, 512, 14336, 4, dict(engine=2, split_k=2, waves=2, row_tiles=2, depth=3))))
     jobs.append(("mid", *gemm(128, 1024, 2048, 5)))
     jobs.append(("mid split-K", *gemm(64, 512, 8192, 6, dict(engine=4, split_k=2, waves=8, row_tiles=2, m_blocks=2, depth=4, k_chunks=2))))
+    # the library's own choices with a K split, several activation tiles, whole tiles per wave and a partial last K block
+    jobs.append(("several activation tiles, two K splits", *gemm(40, 1024, 16384, 9)))
+    jobs.append(("whole tiles per wave", *gemm(8, 20480, 512, 10)))
+    jobs.append(("partial last block", *gemm(8, 2048, 1408, 11)))
+    jobs.append(("partial last block, whole tiles per wave", *gemm(16, 20480, 400, 12)))
+    jobs.append(("partial last block, mid", *gemm(96, 8192, 400, 13)))
 
     a8, vals, meta, _, scale = oracle.make_sparse24_operands(8, 1024, 2048, seed=7)
     sA, sV, sM, sS = dev(a8), dev(vals), dev(meta), scale_tensor(scale)
