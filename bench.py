@@ -60,6 +60,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs (for counter runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies (known traffic, to scale profiler counters)")
+    ap.add_argument("--several-tiles-counters", action="store_true",
+                    help="more than 32 rows on small weight matrices (the skinny ring over several 32-row activation tiles): "
+                         "launch the library's choice three times each on cold weights and exit (for HBM-traffic counters)")
     ap.add_argument("--mid-batch-counters", action="store_true",
                     help="only launch the mid-batch GEMMs (M = 64, 128, 256), eagerly, three times each, and exit "
                          "(for MFMA-utilisation counter runs; prints no JSON line)")
@@ -423,6 +426,21 @@ def main():
                 if rc != 0:
                     raise RuntimeError("sg_sparse24_gemm: %s" % sg.strerror(rc))
             torch.cuda.synchronize()
+        return
+
+    if args.several_tiles_counters:
+        # more than 32 rows on small weight matrices: the skinny ring over several 32-row activation tiles
+        one = torch.ones(1, device="cuda")
+        for (m, n, k) in ((64, 4096, 4096), (128, 2048, 4096), (256, 1024, 4096), (128, 4096, 4096)):
+            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(24)]
+            a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+            d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+            for i in range(3):
+                rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, None)
+                if rc != 0:
+                    raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
+            torch.cuda.synchronize()
+            del wb
         return
 
     if args.k_tail_counters:
