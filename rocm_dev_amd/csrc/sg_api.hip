@@ -456,9 +456,11 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     struct Tile { int bn, bm, waves; };
     // {224, *, 14}: fourteen waves; 57344 = 256 x 224 gives every CU a tile where 256-row tiles fill 224 of 256
     // (5-10 % at M = 128 and 256 on N(0,1)-quantised operands, 4 % at M = 64 over two co-resident 128 x 64 tiles)
-    // The 64 x 128 tile on four waves only where it covers all of m and K is between 4096 and 8192 (stacked - 129..192
-    // or more than 256 rows on a narrow weight matrix, where its padded rows look like a fuller round - 128 x 64 on
-    // eight waves measured 6-12 % faster, ten shapes; at K = 8192 and 96..128 rows 3-8 % faster, three shapes).
+    // The 64 x 128 tile on four waves only where it covers all of m and K is beyond 4096 - up to 96 rows at any such K
+    // that is not a power of two (with rows 8192 bytes apart the eight-wave tile is 3-5 % ahead: 72 x 12288 x 8192 30.5
+    // against 31.8), at 97..128 rows below K = 8192 (stacked - 129..192 or more than 256 rows on a narrow weight matrix, where its padded
+    // rows look like a fuller round - 128 x 64 on eight waves measured 6-12 % faster, ten shapes; at K = 8192 and more
+    // and 96..128 rows 2-8 % faster, nine shapes).
     static const Tile order[] = {{128, 128, 8}, {128, 64, 8}, {64, 64, 4}, {64, 128, 4}, {256, 128, 8}, {224, 128, 14},
                                  {256, 64, 8}, {224, 64, 14}, {128, 256, 8}, {256, 256, 8}, {224, 256, 14}};
     const int bm_max = m <= 64 ? 64 : (m <= 128 ? 128 : 256);
@@ -469,7 +471,7 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     for (const Tile& t : order) {
         if (t.bm > bm_max) continue;
         const bool tall4 = t.bn == 64 && t.bm == 128;
-        if (tall4 && (m > 128 || blocks <= 32 || blocks >= 64)) continue;
+        if (tall4 && (m > 128 || blocks <= 32 || (blocks >= 64 && (m > 96 || (k & (k - 1)) == 0)))) continue;
         const long m_tiles = (m + t.bm - 1) / t.bm;
         const long tiles = (long)((n + t.bn - 1) / t.bn) * m_tiles;
         for (int sk = 1; sk <= 4; sk++) {
@@ -499,10 +501,11 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
                 if (sk == 1 && best.split_k > 1 && wgs * 10 >= rounds * cu_count * 7) better = true;
                 if (sk > 1 && best.split_k == 1 && best_wgs * 10 >= rounds * cu_count * 7) better = false;
             }
-            // 65..128 rows, K of 4224..8064: against 128 x 64 on eight waves and two activation tiles, one 64 x 128 tile
+            // 65..128 rows, K beyond 4096 (from 97 rows on: below 8192): against 128 x 64 on eight waves and two activation tiles, one 64 x 128 tile
             // over all of m on four waves - as many workgroups, the weights pass each CU once (72 x 13824 x 5120
-            // 29.6 -> 23.5 us, 100 rows 28.6 -> 26.1, 72 x 14336 x 5120 28.3 -> 23.7, 72 x 12288 x 5120 28.0 -> 23.0;
-            // level at K = 4096)
+            // 29.6 -> 23.5 us, 100 rows 28.6 -> 26.1, 72 x 14336 x 5120 28.3 -> 23.7, 72 x 12288 x 5120 28.0 -> 23.0,
+            // 72 x 16384 x 11008 59.5 -> 44.1, 72 x 16384 x 14336 73.1 -> 54.1, 72 x 12288 x 10240 52.0 -> 42.4; level at
+            // K = 4096 - the second 64-row activation tile of a 72-row problem re-reads all weights for 8 rows)
             if (tall4 && sk == 1 && rounds == best_rounds && best_tile && best_tile->bn == 128 && best_tile->bm == 64 &&
                 best.split_k == 1 && wgs * 16 >= best_wgs * 15)
                 better = true;
