@@ -494,10 +494,10 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
                           // as full with less splitting, when the splits had become short
                           (rounds == best_rounds && wgs == best_wgs && sk < best.split_k &&
                            blocks / best.split_k < 48);
-            if (best_rounds >= 0 && rounds == best_rounds && blocks < 96 && m > 64) {
-                // above 64 rows and below K = 12288 an unsplit launch that fills 70 % of its rounds beats a split one
+            if (best_rounds >= 0 && rounds == best_rounds && blocks < 80 && m > 64) {
+                // above 64 rows and below K = 10240 an unsplit launch that fills 70 % of its rounds beats a split one
                 // that fills them all (144 x 8192 x 8192: 192 workgroups unsplit 29.1 us, 256 split in two 31.7);
-                // with a longer K the split wins (448 x 4096 x 14336: 46.2 against 50.4)
+                // with a longer K the split wins (448 x 4096 x 14336: 46.2 against 50.4, 200 x 6144 x 11008: 37.9 against 42.9)
                 if (sk == 1 && best.split_k > 1 && wgs * 10 >= rounds * cu_count * 7) better = true;
                 if (sk > 1 && best.split_k == 1 && best_wgs * 10 >= rounds * cu_count * 7) better = false;
             }

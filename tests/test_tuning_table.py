@@ -192,7 +192,7 @@ def test_heuristics_pick_the_fourteen_wave_tile_where_it_fills_the_chip():
 def test_mid_batch_tile_choice_between_the_tile_heights():
     """Row counts that no tile height divides: padded rows are not a fuller round (no stacked 64 x 128 tiles), a split
     whose fp32 partials rival the weights is not taken, an unsplit round that is 70 % full stays unsplit below
-    K = 12288, one 64 x 128 tile covers 65..128 rows when K is beyond 4096, and fourteen-wave tiles of 128 rows or more
+    K = 10240, one 64 x 128 tile covers 65..128 rows when K is beyond 4096, and fourteen-wave tiles of 128 rows or more
     may be stacked.  (tile n, tile m, waves, split) per shape, as measured best or within 2 % of it."""
     want = {(160, 8192, 8192): (128, 64, 8, 1), (144, 6144, 4096): (128, 64, 8, 1), (320, 8192, 8192): (128, 128, 8, 1),
             (144, 4096, 14336): (128, 64, 8, 2), (448, 4096, 14336): (128, 128, 8, 2), (320, 4096, 4096): (128, 64, 8, 1),
