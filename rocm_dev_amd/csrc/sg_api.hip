@@ -493,7 +493,7 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
                           (rounds == best_rounds && wgs * 16 > best_wgs * 17) ||   // clearly fuller round
                           // as full with less splitting, when the splits had become short
                           (rounds == best_rounds && wgs == best_wgs && sk < best.split_k &&
-                           blocks / best.split_k < 48);
+                           blocks / best.split_k < 40);
             if (best_rounds >= 0 && rounds == best_rounds && blocks < 80 && m > 64) {
                 // above 64 rows and below K = 10240 an unsplit launch that fills 70 % of its rounds beats a split one
                 // that fills them all (144 x 8192 x 8192: 192 workgroups unsplit 29.1 us, 256 split in two 31.7);
