@@ -60,6 +60,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs (for counter runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run three 256 MiB device-to-device copies (known traffic, to scale profiler counters)")
+    ap.add_argument("--launch-shapes", nargs="+", metavar="MxNxK",
+                    help="launch the library's own choice for each dense shape three times, eagerly, on rotating cold weight "
+                         "buffers, and exit (for kernel traces and counters of any shape; prints the chosen records)")
     ap.add_argument("--several-tiles-counters", action="store_true",
                     help="more than 32 rows on small weight matrices (the skinny ring over several 32-row activation tiles): "
                          "launch the library's choice three times each on cold weights and exit (for HBM-traffic counters)")
@@ -426,6 +429,25 @@ def main():
                 if rc != 0:
                     raise RuntimeError("sg_sparse24_gemm: %s" % sg.strerror(rc))
             torch.cuda.synchronize()
+        return
+
+    if args.launch_shapes:
+        one = torch.ones(1, device="cuda")
+        for spec in args.launch_shapes:
+            m, n, k = (int(v) for v in spec.lower().split("x"))
+            copies = min(6, max(3, int(COLD_BYTES // (n * k)) + 1))
+            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(copies)]
+            a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+            d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+            t, _ = sg.skinny_gemm_choice(m, n, k)
+            print("%s: %s" % (spec, {f: getattr(t, f) for f in ("engine", "split_k", "waves", "row_tiles", "m_blocks", "depth", "k_chunks",
+                                                                 "persistent_wgs_per_cu", "wave_tiles")}), file=sys.stderr)
+            for i in range(3):
+                rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(), m, n, k, k, None)
+                if rc != 0:
+                    raise RuntimeError("sg_skinny_gemm_auto(%s): %s" % (spec, sg.strerror(rc)))
+            torch.cuda.synchronize()
+            del wb
         return
 
     if args.several_tiles_counters:
