@@ -55,8 +55,8 @@ const char* sg_strerror(int code);
  * device and stream: launches on one stream run in order and share a workspace, launches on different
  * streams may overlap and never share one.  A workspace is created, or grown, by the first launch on its
  * stream that needs it (split_k > 1, also when the library chooses the split itself); at most 512 MB of
- * partials per launch, beyond that SG_WORKSPACE_TOO_SMALL.  An outgrown buffer is kept until the process
- * ends.  A launch recorded into a HIP graph keeps the workspace of the stream it was captured on: run no
+ * partials per launch, beyond that SG_WORKSPACE_TOO_SMALL.  An outgrown buffer is kept until it is released
+ * (below).  A launch recorded into a HIP graph keeps the workspace of the stream it was captured on: run no
  * other split-K work on that stream while the graph replays elsewhere.
  *   sg_init          sets up the current device and a 64 MB workspace for the default stream
  *   sg_init_stream   the same for `stream` with room for partial_bytes of partials, so that later launches
@@ -65,6 +65,30 @@ const char* sg_strerror(int code);
 int    sg_init(void);
 int    sg_init_stream(void* stream, size_t partial_bytes);
 size_t sg_workspace_bytes(void);
+
+/* Giving the library-owned buffers back (split-K workspaces, buffers they have outgrown, the activation scratch of
+ * sg_skinny_gemm_bf16act): sg_release_stream waits for `stream` and frees what the library holds for it on the
+ * current device - call it before destroying a stream, whose handle the runtime may hand out again -;
+ * sg_release_workspaces waits for the device and frees everything, after which sg_workspace_bytes() is 0.  Later
+ * launches allocate afresh.  A HIP graph that recorded a launch keeps pointing at the workspace of its capture
+ * stream: release only after such graphs are destroyed. */
+int    sg_release_stream(void* stream);
+int    sg_release_workspaces(void);
+
+/* The fastpath on caller-owned memory: the reference launcher allocates nothing and keeps no state
+ * (skinny_gemm/skinny_gemm_caller.cu:20-43; the caller owns even the one-word scale, skinny_gemm/test.cu:78-79), and
+ * sg_skinny_gemm_auto_ws does the same - its split-K partials and arrival counters live in `workspace` and nowhere
+ * else, nothing is allocated, and a launch that would need more than it is given returns SG_WORKSPACE_TOO_SMALL.
+ *   sg_workspace_query  *bytes = what sg_skinny_gemm_auto_ws needs for the shape with the tuning table as it is now
+ *                       (0 when the launch it would choose has no K split; then workspace may be NULL)
+ *   sg_workspace_init   zeroes the counter region (the first 64 KB) of a workspace with a kernel in stream order:
+ *                       once per buffer, before its first use; every launch that completes leaves it zero again
+ * workspace: device memory, 256-byte aligned, [16384 arrival counters][fp32 partials]; one buffer serves launches of
+ * different shapes in stream order (size it by the largest query); launches that overlap need a buffer each. */
+int sg_workspace_query(int m, int n, int k, size_t* bytes);
+int sg_workspace_init(void* workspace, size_t bytes, void* stream);
+int sg_skinny_gemm_auto_ws(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
+                           int m, int n, int k, int b_stride, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Dense FP8 skinny GEMM:  D[m,n] = bf16( scale[0] * sum_k A[m,k] * B[n,k] ).
@@ -149,7 +173,10 @@ typedef struct SgTuning {
                           (all need persistent_wgs_per_cu >= 1, split_k = 1, m <= 16*m_blocks); + 4 = persistent
                           workgroups get one extra wavefront that streams nothing and does every reduction and store;
                           8 (alone, with row_tiles = 2, m_blocks = 1, persistent_wgs_per_cu = 0) = 24-row tiles: the
-                          second 16-row fragment carries 8 weight rows (6144 rows = 256 tiles instead of 384) */
+                          second 16-row fragment carries 8 weight rows (6144 rows = 256 tiles instead of 384);
+                          mid-batch: 0 = the last workgroup of a tile to arrive sums the tile's split_k partials, 1 = the
+                          GEMM launch stores partials only and a second launch sums them, one wave per 16 x 16 fragment
+                          over the whole device (same split order, same result bits); anything else is SG_INVALID_CONFIG */
 } SgTuning;
 
 int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
@@ -161,7 +188,8 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const
  * device image (8 MB + 4096 counters per GPU, held until the process ends) instead of a workspace from
  * hipMalloc, and nothing is allocated or freed by the call.  A configuration whose partials need more
  * (tiles * split_k * fragment bytes > 8 MB, or more than 4096 output tiles with split_k > 1) is refused
- * with SG_WORKSPACE_TOO_SMALL; without a K split there is no limit.  All calls on one GPU share the array:
+ * with SG_WORKSPACE_TOO_SMALL; without a K split there is no limit.  The counters are cleared by a kernel with
+ * the first call on a device; after that every launch that completes leaves them zero.  All calls on one GPU share the array:
  * calls that overlap on one GPU (two streams, unordered graph nodes) race, calls in stream order do not. */
 int sg_skinny_gemm_tuned_noalloc(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,
                                  int m, int n, int k, int b_stride, const SgTuning* tuning, void* stream);
@@ -212,6 +240,11 @@ int sg_skinny_gemm_choice(int m, int n, int k, SgTuning* out, int* from_table);
  * heuristics.  A record the kernels cannot run for the shape (no such instantiation, ring larger than
  * LDS, ...) is skipped at launch and the heuristics' choice runs.  The table is process-wide and may be
  * read and changed from any thread; a launch uses the table as it is when the launch is made.
+ * The library ships the table its tuning driver found for the benchmark shapes on MI355X
+ * (rocm_dev_amd/tuning/mi355x.tbl, looked for as ../tuning/mi355x.tbl from the directory of libsgemm.so) and merges
+ * it into the table once, before the table is first read or changed - the counterpart of the reference committing
+ * what its search found (skinny_gemm/core.cu:29-38).  The environment variable SGEMM_TUNING_TABLE names another file
+ * to load instead; empty or "none" starts with an empty table.
  *   sg_tuning_set    stores a copy of *t for the shape (engine 1, 2 or 4); t == NULL removes the entry
  *   sg_tuning_get    SG_SUCCESS and *out, or SG_INVALID_CONFIG when the table has no entry
  *   sg_tuning_load   merges a file into the table; SG_BAD_ARGUMENT (table unchanged) if the file cannot be
@@ -225,23 +258,6 @@ int sg_tuning_count(void);
 int sg_tuning_clear(void);
 int sg_tuning_load(const char* path);
 int sg_tuning_save(const char* path);
-
-/* Profiling aid, no counterpart in the reference.  While a buffer is set, every launch of the LDS-ring GEMM
- * kernels (per-tile and persistent) takes the next grid * 8 words of it and each workgroup leaves eight 64-bit
- * words there when it is done: [0] kernel entry, [1] prologue DMAs issued, [2] first stage landed, [3] last stage
- * consumed, [4] outputs stored and acknowledged - 10 ns ticks of the device's constant 100 MHz clock -
- * [5], [6] shader clock at entry and end, [7] XCC_ID << 32 | HW_ID.  Launches that no longer fit leave nothing.
- * A launch recorded into a HIP graph keeps its slice on every replay.  Process-wide; set it from one thread while
- * no other thread launches.  sg_debug_stamps(NULL, 0) switches the stamps off again. */
-int sg_debug_stamps(unsigned long long* device_buffer, size_t n_words);
-
-/* Profiling aid, no counterpart in the reference: reads the n x k weight matrix B (row stride b_stride, k % 1024 == 0)
- * the way the persistent LDS-ring GEMM streams it - one workgroup per CU walking row tiles, eight waves sharing K,
- * direct-to-LDS loads with the streaming hint, two 4 KB slots per wave - and does nothing with it.  Its duration is the
- * ceiling of that access pattern on the device: what a GEMM's streaming phase is measured against.  segment_bytes is
- * what one load instruction takes contiguously from one row: 256 (4 rows per instruction - the GEMM's own pattern),
- * 512 (2 rows) or 1024 (1 row). */
-int sg_debug_read_stream(const uint8_t* B, int n, int k, int b_stride, int segment_bytes, void* stream);
 
 /* Replaces  template<class out> void async_gemm(const fp8* A, const fp8* B, out* D, int m,
  * int n, int k)  (async_gemm_sparse/sparse_k.cu:45-69, async_gemm_blanes/sparse_k.cu,

@@ -26,6 +26,11 @@ from .api import (  # noqa: F401
     skinny_gemm_tuned_noalloc,
     init_stream,
     workspace_bytes,
+    workspace_query,
+    workspace_init,
+    skinny_gemm_auto_ws,
+    release_stream,
+    release_workspaces,
     strerror,
     tiled_sum_reduce,
     tuning_clear,

@@ -1,4 +1,4 @@
-"""Loads libsgemm.so and declares the C ABI of include/sgemm.h to ctypes.
+"""Loads libsgemm.so and declares the C ABI of include/sgemm.h (and the profiling aids of include/sgemm_debug.h) to ctypes.
 
 There is no fallback: if the library has not been built the import fails loudly.
 """
@@ -21,6 +21,11 @@ SIGNATURES = {
     "sg_init": (_i, []),
     "sg_init_stream": (_i, [_vp, _sz]),
     "sg_workspace_bytes": (_sz, []),
+    "sg_release_stream": (_i, [_vp]),
+    "sg_release_workspaces": (_i, []),
+    "sg_workspace_query": (_i, [_i, _i, _i, C.POINTER(_sz)]),
+    "sg_workspace_init": (_i, [_vp, _sz, _vp]),
+    "sg_skinny_gemm_auto_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
     "sg_debug_stamps": (_i, [_vp, _sz]),
     "sg_debug_read_stream": (_i, [_vp, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),

@@ -65,13 +65,66 @@ def _dev(t, *dtypes):
 _FP8 = (torch.uint8, torch.float8_e4m3fn)
 
 
+# The C ABI takes raw pointers with the shapes it is told: everything it will assume about a tensor is checked here,
+# before the call - a transposed or sliced operand would otherwise be read with the wrong strides, and a weight matrix
+# with fewer columns than k past its allocation.
+def _same_device(*tensors):
+    live = [t for t in tensors if t is not None]
+    for t in live:
+        if not t.is_cuda:
+            raise ValueError("expected CUDA (HIP) tensors")
+        if t.device != live[0].device:
+            raise ValueError("operands on different devices: %s and %s" % (live[0].device, t.device))
+
+
+def _row_major(t, name):
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous (row-major), got strides %s for shape %s"
+                         % (name, tuple(t.stride()), tuple(t.shape)))
+
+
+def _weights(B, cols, name="B"):
+    """[n, cols] with the columns contiguous; rows may be further apart than cols (a row stride)."""
+    if B.dim() != 2 or B.shape[1] != cols:
+        raise ValueError("%s must be [n, %d], got %s" % (name, cols, tuple(B.shape)))
+    if B.shape[1] > 1 and B.stride(1) != 1:
+        raise ValueError("%s must have contiguous columns, got strides %s" % (name, tuple(B.stride())))
+    if B.shape[0] > 1 and B.stride(0) < cols:
+        raise ValueError("%s: row stride %d below its %d columns" % (name, B.stride(0), cols))
+    return B.stride(0) if B.shape[0] > 1 else max(B.stride(0), cols)
+
+
+def _gemm_operands(A, B, D, scale_tensor=None, weight_cols=None, extra=()):
+    """(m, n, k, b_stride) of D[m, n] = A[m, k] x B[n, weight_cols or k]^T after checking every layout assumption."""
+    if A.dim() != 2 or D.dim() != 2:
+        raise ValueError("A and D must be 2-D, got %s and %s" % (tuple(A.shape), tuple(D.shape)))
+    m, k = A.shape
+    b_stride = _weights(B, k if weight_cols is None else weight_cols)
+    n = B.shape[0]
+    if tuple(D.shape) != (m, n):
+        raise ValueError("D must be [%d, %d], got %s" % (m, n, tuple(D.shape)))
+    _row_major(A, "A")
+    _row_major(D, "D")
+    if scale_tensor is not None and (scale_tensor.numel() < 1 or not scale_tensor.is_contiguous()):
+        raise ValueError("scale_tensor must hold at least one float")
+    _same_device(A, B, D, scale_tensor, *extra)
+    return m, n, k, b_stride
+
+
+def _vector(t, length, name):
+    if t is not None and (tuple(t.shape) != (length,) or not t.is_contiguous()):
+        raise ValueError("%s must be a contiguous vector of %d floats, got shape %s strides %s"
+                         % (name, length, tuple(t.shape), tuple(t.stride())))
+
+
 def skinny_gemm(A, B, D, scale_tensor, split_k, A_producers, B_producers, consumers, b_lanes, qsize, op_m, ops,
                 b_stride=None, check=False):
     """D[m,n] = bf16(scale * A[m,k] @ B[n,k]^T) with explicit tunables.  B is [n, k] with row stride b_stride."""
-    m, k = A.shape
-    n = B.shape[0]
+    m, n, k, row_stride = _gemm_operands(A, B, D, scale_tensor)
     if b_stride is None:
-        b_stride = B.stride(0)
+        b_stride = row_stride
+    elif n > 1 and b_stride != row_stride:
+        raise ValueError("b_stride %d is not the row stride of B (%d)" % (b_stride, row_stride))
     with torch.cuda.device(A.device):
         rc = lib.sg_skinny_gemm(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
                                 _dev(scale_tensor, torch.float32), m, n, k, b_stride, split_k, A_producers,
@@ -81,11 +134,10 @@ def skinny_gemm(A, B, D, scale_tensor, split_k, A_producers, B_producers, consum
 
 def skinny_gemm_fastpath(A, B, D, scale_tensor, check=False):
     """Library-chosen configuration; B is [n, k] (row stride taken from the tensor)."""
-    m, k = A.shape
-    n = B.shape[0]
+    m, n, k, b_stride = _gemm_operands(A, B, D, scale_tensor)
     with torch.cuda.device(A.device):
         rc = lib.sg_skinny_gemm_auto(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
-                                     _dev(scale_tensor, torch.float32), m, n, k, B.stride(0), _stream())
+                                     _dev(scale_tensor, torch.float32), m, n, k, b_stride, _stream())
     return _done(rc, check)
 
 
@@ -106,18 +158,15 @@ def tuning_as_dict(t):
 
 def skinny_gemm_rowcol(A, B, D, scale_tensor=None, row_scales=None, col_scales=None, check=False):
     """D = bf16(((A @ B^T) * scale) * row_scales[:, None] * col_scales[None, :]); any factor may be None."""
-    m, k = A.shape
-    n = B.shape[0]
-    if row_scales is not None and tuple(row_scales.shape) != (m,):
-        raise ValueError("row_scales must have shape (m,)")
-    if col_scales is not None and tuple(col_scales.shape) != (n,):
-        raise ValueError("col_scales must have shape (n,)")
+    m, n, k, b_stride = _gemm_operands(A, B, D, scale_tensor, extra=(row_scales, col_scales))
+    _vector(row_scales, m, "row_scales")
+    _vector(col_scales, n, "col_scales")
     with torch.cuda.device(A.device):
         rc = lib.sg_skinny_gemm_rowcol(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
                                        None if scale_tensor is None else _dev(scale_tensor, torch.float32),
                                        None if row_scales is None else _dev(row_scales, torch.float32),
                                        None if col_scales is None else _dev(col_scales, torch.float32),
-                                       m, n, k, B.stride(0), _stream())
+                                       m, n, k, b_stride, _stream())
     return _done(rc, check)
 
 
@@ -126,16 +175,13 @@ def skinny_gemm_bf16act(X, B, D, scale_tensor=None, col_scales=None, row_scales_
     D = bf16(((q(X) @ B^T) * scale) * row_scale[:, None] * col_scales[None, :]); row_scales_out, if given, receives the
     row scales.  One launch where the fused kernel pays (skinny_gemm_bf16act_choice), two inside the library otherwise;
     with `tuning` (an SgTuning; engine 0 = the library's record for the shape) always the fused kernel."""
-    m, k = X.shape
-    n = B.shape[0]
-    if col_scales is not None and tuple(col_scales.shape) != (n,):
-        raise ValueError("col_scales must have shape (n,)")
-    if row_scales_out is not None and tuple(row_scales_out.shape) != (m,):
-        raise ValueError("row_scales_out must have shape (m,)")
+    m, n, k, b_stride = _gemm_operands(X, B, D, scale_tensor, extra=(col_scales, row_scales_out))
+    _vector(col_scales, n, "col_scales")
+    _vector(row_scales_out, m, "row_scales_out")
     args = (_dev(X, torch.bfloat16), _dev(B, *_FP8), _dev(D, torch.bfloat16),
             None if scale_tensor is None else _dev(scale_tensor, torch.float32),
             None if col_scales is None else _dev(col_scales, torch.float32),
-            None if row_scales_out is None else _dev(row_scales_out, torch.float32), m, n, k, B.stride(0))
+            None if row_scales_out is None else _dev(row_scales_out, torch.float32), m, n, k, b_stride)
     with torch.cuda.device(X.device):
         if tuning is None:
             rc = lib.sg_skinny_gemm_bf16act(*args, _stream())
@@ -156,14 +202,13 @@ def skinny_gemm_bf16act_choice(m, n, k):
 def skinny_gemm_tuned(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k=1, waves=4, row_tiles=1, m_blocks=None,
                       depth=2, k_chunks=4, non_temporal=1, persistent_wgs_per_cu=0, wave_tiles=0, check=False):
     """The library-native tuning entry (no reference counterpart): pick the engine and its shape."""
-    m, k = A.shape
-    n = B.shape[0]
+    m, n, k, b_stride = _gemm_operands(A, B, D, scale_tensor)
     if m_blocks is None:
         m_blocks = 1 if m <= 16 else 2
     t = SgTuning(engine, split_k, waves, row_tiles, m_blocks, depth, k_chunks, non_temporal, persistent_wgs_per_cu, wave_tiles)
     with torch.cuda.device(A.device):
         rc = lib.sg_skinny_gemm_tuned(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
-                                      _dev(scale_tensor, torch.float32), m, n, k, B.stride(0), C.byref(t), _stream())
+                                      _dev(scale_tensor, torch.float32), m, n, k, b_stride, C.byref(t), _stream())
     return _done(rc, check)
 
 
@@ -171,14 +216,13 @@ def skinny_gemm_tuned_noalloc(A, B, D, scale_tensor, engine=ENGINE_AUTO, split_k
                               depth=2, k_chunks=4, non_temporal=1, persistent_wgs_per_cu=0, wave_tiles=0, check=False):
     """skinny_gemm_tuned with the split-K partials in the library's fixed device array: allocates nothing, refuses
     configurations whose partials exceed 8 MB or 4096 tiles with WORKSPACE_TOO_SMALL (no reference counterpart)."""
-    m, k = A.shape
-    n = B.shape[0]
+    m, n, k, b_stride = _gemm_operands(A, B, D, scale_tensor)
     if m_blocks is None:
         m_blocks = 1 if m <= 16 else 2
     t = SgTuning(engine, split_k, waves, row_tiles, m_blocks, depth, k_chunks, non_temporal, persistent_wgs_per_cu, wave_tiles)
     with torch.cuda.device(A.device):
         rc = lib.sg_skinny_gemm_tuned_noalloc(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
-                                              _dev(scale_tensor, torch.float32), m, n, k, B.stride(0), C.byref(t),
+                                              _dev(scale_tensor, torch.float32), m, n, k, b_stride, C.byref(t),
                                               _stream())
     return _done(rc, check)
 
@@ -191,6 +235,45 @@ def init_stream(stream=None, partial_bytes=64 << 20, check=True):
 
 def workspace_bytes():
     return lib.sg_workspace_bytes()
+
+
+def release_stream(stream=None, check=True):
+    """Wait for `stream` (torch stream; None = torch's current stream) and free what the library holds for it."""
+    handle = _stream() if stream is None else stream.cuda_stream
+    return _done(lib.sg_release_stream(handle), check)
+
+
+def release_workspaces(check=True):
+    """Wait for the device and free every buffer the library owns on it; workspace_bytes() is 0 afterwards."""
+    return _done(lib.sg_release_workspaces(), check)
+
+
+def workspace_query(m, n, k):
+    """Bytes of caller-owned workspace skinny_gemm_auto_ws needs for the shape (0: the launch has no K split)."""
+    need = C.c_size_t(0)
+    rc = lib.sg_workspace_query(m, n, k, C.byref(need))
+    if rc != 0:
+        raise SgError(rc)
+    return need.value
+
+
+def workspace_init(workspace, check=True):
+    """Clear the counter region of a caller-owned workspace (a uint8 CUDA tensor) in stream order: once per buffer."""
+    return _done(lib.sg_workspace_init(_dev(workspace, torch.uint8), workspace.numel(), _stream()), check)
+
+
+def skinny_gemm_auto_ws(A, B, D, scale_tensor, workspace=None, check=False):
+    """skinny_gemm_fastpath on caller-owned memory: `workspace` (uint8 CUDA tensor, 256-byte aligned, prepared once with
+    workspace_init; None where workspace_query says 0) holds the split-K partials and counters, nothing is allocated."""
+    m, n, k, b_stride = _gemm_operands(A, B, D, scale_tensor, extra=(workspace,))
+    if workspace is not None:
+        _row_major(workspace, "workspace")
+    with torch.cuda.device(A.device):
+        rc = lib.sg_skinny_gemm_auto_ws(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
+                                        _dev(scale_tensor, torch.float32), m, n, k, b_stride,
+                                        None if workspace is None else _dev(workspace, torch.uint8),
+                                        0 if workspace is None else workspace.numel(), _stream())
+    return _done(rc, check)
 
 
 def skinny_gemm_pick(m, n, k):
@@ -255,9 +338,18 @@ class HFRK_skinny_gemm:
 
     def skinny_gemm_torch_binding(self, A, B, D, scale_tensor, split_k, A_producers, B_producers, consumers,
                                   b_lanes, qsize, ops):
+        # B arrives as the (K, N) view of an N x K, K-contiguous weight matrix (skinny_gemm_binding.cu:36-41)
+        if A.dim() != 2 or B.dim() != 2 or B.size(0) != A.size(1) or tuple(D.shape) != (A.size(0), B.size(1)):
+            raise ValueError("A [m, k], B [k, n] (a view of n x k weights) and D [m, n] disagree: %s %s %s"
+                             % (tuple(A.shape), tuple(B.shape), tuple(D.shape)))
+        if (B.size(0) > 1 and B.stride(0) != 1) or (B.size(1) > 1 and B.stride(1) < B.size(0)):
+            raise ValueError("B must be the transposed view of K-contiguous weights, got strides %s" % (tuple(B.stride()),))
+        _row_major(A, "A")
+        _row_major(D, "D")
+        _same_device(A, B, D, scale_tensor)
         m, k = A.size(0), A.size(1)
         n = B.size(1)
-        b_stride = B.stride(1)
+        b_stride = B.stride(1) if n > 1 else max(B.stride(1), k)
         op_m = 8 if m <= 8 else (16 if m <= 16 else 32)
         with torch.cuda.device(A.device):
             return lib.sg_skinny_gemm(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D, torch.bfloat16),
@@ -267,8 +359,12 @@ class HFRK_skinny_gemm:
 
 def sparse24_gemm(A, B_vals, B_meta, D, scale_tensor, tuning=None, check=False):
     """2:4 sparse weights: B_vals [n, k/2] kept codes, B_meta [n, k/8] position nibbles (include/sgemm.h)."""
-    m, k = A.shape
-    n = B_vals.shape[0]
+    if A.dim() != 2 or A.shape[1] % 8:
+        raise ValueError("A must be [m, k] with k a multiple of 8, got %s" % (tuple(A.shape),))
+    m, n, k, _ = _gemm_operands(A, B_vals, D, scale_tensor, weight_cols=A.shape[1] // 2, extra=(B_meta,))
+    _row_major(B_vals, "B_vals")
+    if tuple(B_meta.shape) != (n, k // 8) or not B_meta.is_contiguous():
+        raise ValueError("B_meta must be a contiguous [%d, %d], got %s" % (n, k // 8, tuple(B_meta.shape)))
     with torch.cuda.device(A.device):
         if tuning is None:
             rc = lib.sg_sparse24_gemm(_dev(A, *_FP8), _dev(B_vals, *_FP8), _dev(B_meta, torch.uint8),
@@ -283,17 +379,25 @@ def sparse24_gemm(A, B_vals, B_meta, D, scale_tensor, tuning=None, check=False):
 def sparse24_compress(B, B_vals, B_meta, check=False):
     """Prune dense E4M3 weights B [n, k] to 2:4 (two largest magnitudes per group of four) and compress them
     into B_vals [n, k/2] and B_meta [n, k/8] (format of include/sgemm.h)."""
+    if B.dim() != 2 or B.shape[1] % 8:
+        raise ValueError("B must be [n, k] with k a multiple of 8, got %s" % (tuple(B.shape),))
     n, k = B.shape
+    b_stride = _weights(B, k)
+    if tuple(B_vals.shape) != (n, k // 2) or tuple(B_meta.shape) != (n, k // 8):
+        raise ValueError("B_vals must be [%d, %d] and B_meta [%d, %d]" % (n, k // 2, n, k // 8))
+    _row_major(B_vals, "B_vals")
+    _row_major(B_meta, "B_meta")
+    _same_device(B, B_vals, B_meta)
     with torch.cuda.device(B.device):
-        rc = lib.sg_sparse24_compress(_dev(B, *_FP8), _dev(B_vals, *_FP8), _dev(B_meta, torch.uint8), n, k, B.stride(0),
+        rc = lib.sg_sparse24_compress(_dev(B, *_FP8), _dev(B_vals, *_FP8), _dev(B_meta, torch.uint8), n, k, b_stride,
                                       _stream())
     return _done(rc, check)
 
 
 def async_gemm(A, B, D, check=False):
     """D = A @ B^T without a scale on the default stream; D is float32 or bfloat16."""
-    m, k = A.shape
-    n = B.shape[0]
+    m, n, k, _ = _gemm_operands(A, B, D)
+    _row_major(B, "B")
     with torch.cuda.device(A.device):
         if D.dtype == torch.float32:
             rc = lib.sg_async_gemm_f32(_dev(A, *_FP8), _dev(B, *_FP8), _dev(D), m, n, k)
@@ -305,6 +409,11 @@ def async_gemm(A, B, D, check=False):
 def tiled_sum_reduce(A, B, D, check=False, lds_queue=False):
     """D[m,n] = sum_b (A[b,m,n] + B[b,m,n]) in fp32, batch order.  lds_queue=True runs the variant that stages the
     batches through a queue in LDS (tiled_sum_reduce_async/src.cu:179-200); the result bits are the same."""
+    if A.dim() != 3 or B.shape != A.shape or tuple(D.shape) != tuple(A.shape[1:]):
+        raise ValueError("A and B must be [b, m, n] and D [m, n], got %s, %s, %s" % (tuple(A.shape), tuple(B.shape), tuple(D.shape)))
+    for t, name in ((A, "A"), (B, "B"), (D, "D")):
+        _row_major(t, name)
+    _same_device(A, B, D)
     b, m, n = A.shape
     fn = lib.sg_tiled_sum_reduce_async if lds_queue else lib.sg_tiled_sum_reduce
     with torch.cuda.device(A.device):
@@ -312,7 +421,19 @@ def tiled_sum_reduce(A, B, D, check=False, lds_queue=False):
     return _done(rc, check)
 
 
+def _codec_operands(X, Q, scales, nbuf=None):
+    if X.dim() != 2 or tuple(Q.shape) != ((tuple(X.shape) if nbuf is None else (nbuf,) + tuple(X.shape))):
+        raise ValueError("row-codec operands must agree in shape, got %s and %s" % (tuple(X.shape), tuple(Q.shape)))
+    want = (X.shape[0],) if nbuf is None else (nbuf, X.shape[0])
+    if tuple(scales.shape) != want:
+        raise ValueError("scales must have shape %s, got %s" % (want, tuple(scales.shape)))
+    for t, name in ((X, "the bf16 matrix"), (Q, "Q"), (scales, "scales")):
+        _row_major(t, name)
+    _same_device(X, Q, scales)
+
+
 def fp8_encode_rows(X, Q, scales, check=False):
+    _codec_operands(X, Q, scales)
     rows, cols = X.shape
     with torch.cuda.device(X.device):
         rc = lib.sg_fp8_encode_rows(_dev(X, torch.bfloat16), _dev(Q, *_FP8), _dev(scales, torch.float32),
@@ -321,6 +442,7 @@ def fp8_encode_rows(X, Q, scales, check=False):
 
 
 def fp8_decode_rows(Q, scales, Y, check=False):
+    _codec_operands(Y, Q, scales)
     rows, cols = Q.shape
     with torch.cuda.device(Q.device):
         rc = lib.sg_fp8_decode_rows(_dev(Q, *_FP8), _dev(scales, torch.float32), _dev(Y, torch.bfloat16),
@@ -330,6 +452,9 @@ def fp8_decode_rows(Q, scales, Y, check=False):
 
 def fp8_reduce_rows(Q, scales, Y, check=False):
     """Q [nbuf, rows, cols], scales [nbuf, rows] -> Y [rows, cols] bfloat16."""
+    if Q.dim() != 3:
+        raise ValueError("Q must be [nbuf, rows, cols], got %s" % (tuple(Q.shape),))
+    _codec_operands(Y, Q, scales, nbuf=Q.shape[0])
     nbuf, rows, cols = Q.shape
     with torch.cuda.device(Q.device):
         rc = lib.sg_fp8_reduce_rows(_dev(Q, *_FP8), _dev(scales, torch.float32), _dev(Y, torch.bfloat16),

@@ -35,6 +35,8 @@ PRESETS = {
     "mid": [(m, n, k) for m in (64, 128, 256)
             for (n, k) in ((10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672))],
 }
+# every dense benchmark shape: what the shipped table (rocm_dev_amd/tuning/mi355x.tbl) is tuned on
+PRESETS["baseline"] = PRESETS["decode"] + PRESETS["mid"]
 
 
 def record(engine, split_k=1, waves=1, row_tiles=1, m_blocks=1, depth=2, k_chunks=4, non_temporal=1,
@@ -111,7 +113,8 @@ def mid_fits(k, r):
     wn = r["waves"] // 2
     dx = r["k_chunks"] if 2 <= r["k_chunks"] < r["depth"] else r["depth"]
     bn, bm = 16 * r["row_tiles"] * wn, 32 * r["m_blocks"]
-    if (r["depth"] * bn + dx * bm) * 128 + (16 if r["split_k"] > 1 else 0) > LDS_BYTES:
+    # (a split whose sum is a second launch, wave_tiles = 1, needs no arrival word)
+    if (r["depth"] * bn + dx * bm) * 128 + (16 if r["split_k"] > 1 and r["wave_tiles"] != 1 else 0) > LDS_BYTES:
         return False
     blocks = k // 128
     return r["split_k"] == 1 or blocks // r["split_k"] >= 8
@@ -129,9 +132,10 @@ def search_space(m, n, k):
                 continue
             if 32 * mb >= 2 * m and mb > 2:      # tile more than twice as tall as the problem
                 continue
-            r = record(ENGINE_MID, sk, waves, rt, mb, depth, dx if dx else depth)
-            if mid_fits(k, r):
-                out.append(r)
+            for wt in ((0,) if sk == 1 else (0, 1)):   # a split's sum by the last workgroup to arrive, or by a second launch
+                r = record(ENGINE_MID, sk, waves, rt, mb, depth, dx if dx else depth, 1, 0, wt)
+                if mid_fits(k, r):
+                    out.append(r)
         # the skinny LDS ring over several 32-row activation tiles (what the library runs on small weight matrices)
         if m <= 256 and (k % 256 == 0 or (k % 16 == 0 and k > 256)):
             for sk, waves, rt, depth in itertools.product((1, 2), (1, 2, 3, 4), (1, 2, 4), (2, 3, 4)):

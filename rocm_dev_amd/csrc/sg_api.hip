@@ -1,5 +1,7 @@
 // C ABI of libsgemm.so: argument validation, configuration choice and launches.
 // The contract of every entry point is documented in include/sgemm.h.
+#include <dlfcn.h>
+
 #include <atomic>
 #include <cstdio>
 #include <cstdlib>
@@ -7,6 +9,7 @@
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "sg_host.h"
 #include "sg_stream_kernel.h"
@@ -38,6 +41,10 @@ static std::mutex g_mutex;
 // their partials and arrival counters; launches on different streams may overlap and must not.
 static std::map<hipStream_t, Workspace> g_ws[kMaxDevices];
 static size_t g_ws_bytes[kMaxDevices];   // device memory held by the workspaces of a device (retired buffers included)
+// Buffers a workspace has outgrown: launches already enqueued may still use them, so they are only freed by
+// sg_release_workspaces / sg_release_stream, behind a synchronisation.
+struct Retired { hipStream_t stream; void* p; size_t bytes; };
+static std::vector<Retired> g_retired[kMaxDevices];
 static DeviceInfo g_dev[kMaxDevices];
 static bool g_dev_known[kMaxDevices];
 
@@ -107,6 +114,33 @@ static int fill_zero(unsigned* p, size_t n, hipStream_t stream) {
     return SG_SUCCESS;
 }
 
+// Zeroes n words of a buffer that nothing uses yet, now: on a stream of the library's own (non-blocking, so it
+// neither joins nor disturbs a capture in progress on the caller's stream), waited for before returning.
+static int fill_zero_now(unsigned* p, size_t n) {
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    hipStream_t own = nullptr;
+    int rc = SG_LAUNCH_FAILED;
+    if (report_hip("hipStreamCreateWithFlags", hipStreamCreateWithFlags(&own, hipStreamNonBlocking)) == hipSuccess) {
+        rc = fill_zero(p, n, own);
+        if (rc == SG_SUCCESS && report_hip("hipStreamSynchronize", hipStreamSynchronize(own)) != hipSuccess) rc = SG_LAUNCH_FAILED;
+        (void)hipStreamDestroy(own);
+    } else {
+        (void)hipGetLastError();
+    }
+    if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode);
+    return rc;
+}
+
+static bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
 // The workspace of `stream` on the current device, grown to hold partial_bytes of fp32 partials and
 // n_counters arrival counters.  A buffer that is outgrown is kept until the process ends (launches
 // already enqueued may still use it); sizes double, so what is kept is less than what is in use.
@@ -120,6 +154,7 @@ int get_workspace(hipStream_t stream, size_t partial_bytes, size_t n_counters, W
         const size_t bytes = round_up_pow2(partial_bytes, kMinPartialBytes);
         void* p = workspace_alloc(bytes);
         if (!p) return SG_NO_DEVICE;
+        if (w.partials) g_retired[dev].push_back({stream, w.partials, w.partial_bytes});
         w.partials = static_cast<float*>(p);
         w.partial_bytes = bytes;
         g_ws_bytes[dev] += bytes;
@@ -128,11 +163,16 @@ int get_workspace(hipStream_t stream, size_t partial_bytes, size_t n_counters, W
         const size_t n = round_up_pow2(n_counters, kMinCounters);
         void* c = workspace_alloc(n * sizeof(unsigned));
         if (!c) return SG_NO_DEVICE;
-        // in stream order before the launch that asked for them (and every later one on this stream)
-        if (int rc = fill_zero(static_cast<unsigned*>(c), n, stream)) {
+        // Zero before the launch that asked for them (and every later one on this stream): in stream order - unless the
+        // stream is being captured, where a kernel launched on it would only be recorded: then at once, outside the
+        // graph, so that the graph's replays and eager launches on the stream alike find the counters zero.
+        const int rc = stream_is_capturing(stream) ? fill_zero_now(static_cast<unsigned*>(c), n)
+                                                   : fill_zero(static_cast<unsigned*>(c), n, stream);
+        if (rc) {
             (void)hipFree(c);
             return rc;
         }
+        if (w.counters) g_retired[dev].push_back({stream, w.counters, w.n_counters * sizeof(unsigned)});
         w.counters = static_cast<unsigned*>(c);
         w.n_counters = n;
         g_ws_bytes[dev] += n * sizeof(unsigned);
@@ -150,10 +190,12 @@ constexpr size_t kStaticCounters = 4096;
 static __device__ __align__(256) unsigned char scratch[kStaticPartialBytes + kStaticCounters * sizeof(unsigned)];
 static unsigned char* g_scratch_ptr[kMaxDevices];   // device address of `scratch` per device, looked up once
 
-static int static_workspace(Workspace* out) {
+// *first_use is set when this call looked the address up (the first call on the device).
+static int static_workspace(Workspace* out, bool* first_use) {
     int dev;
     if (int rc = current_device(&dev)) return rc;
     std::lock_guard<std::mutex> lock(g_mutex);
+    *first_use = false;
     if (!g_scratch_ptr[dev]) {
         void* ptr = nullptr;
         if (report_hip("hipGetSymbolAddress", hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))) != hipSuccess || !ptr) {
@@ -161,6 +203,7 @@ static int static_workspace(Workspace* out) {
             return SG_NO_DEVICE;
         }
         g_scratch_ptr[dev] = static_cast<unsigned char*>(ptr);
+        *first_use = true;
     }
     out->partials = reinterpret_cast<float*>(g_scratch_ptr[dev]);
     out->partial_bytes = kStaticPartialBytes;
@@ -172,9 +215,11 @@ static int static_workspace(Workspace* out) {
 // ---- time stamps (profiling aid) -------------------------------------------------------------------
 static unsigned long long* g_stamp_buf = nullptr;
 static size_t g_stamp_words = 0, g_stamp_cursor = 0;
+static std::atomic<bool> g_stamps_on{false};   // the launch path takes the lock below only while a buffer is set
 
 // Room for one launch of `grid` workgroups, or nullptr when stamps are off or the buffer is full.
 static unsigned long long* take_stamps(unsigned grid) {
+    if (!g_stamps_on.load(std::memory_order_relaxed)) return nullptr;
     std::lock_guard<std::mutex> lock(g_mutex);
     const size_t need = (size_t)grid * kStampWords;
     if (!g_stamp_buf || g_stamp_cursor + need > g_stamp_words) return nullptr;
@@ -440,9 +485,14 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
     set_reciprocals(a);
     // c.ku: ring slots of the activations (0 or out of range = as many as the weights')
     const int dx = (c.ku >= 2 && c.ku < c.depth) ? c.ku : c.depth;
-    const size_t lds = ((size_t)c.depth * bn + (size_t)dx * bm) * 128 + (c.split_k > 1 ? 16 : 0);
+    // c.wavetile = 1: the split-K partials are summed by a second launch over the whole device instead of by the last
+    // workgroup of every tile to arrive (no arrival word in LDS, no counters touched)
+    if (c.wavetile != 0 && c.wavetile != 1) return SG_INVALID_CONFIG;
+    a.defer_reduce = (c.wavetile == 1 && c.split_k > 1) ? 1 : 0;
+    const size_t lds = ((size_t)c.depth * bn + (size_t)dx * bm) * 128 + ((c.split_k > 1 && !a.defer_reduce) ? 16 : 0);
     if (lds > 160 * 1024) return SG_INVALID_CONFIG;
-    return launch_mid(c.rg, c.mt, c.depth, dx, wn, a, (unsigned)(tiles * c.split_k), lds, stream);
+    if (int rc = launch_mid(c.rg, c.mt, c.depth, dx, wn, a, (unsigned)(tiles * c.split_k), lds, stream)) return rc;
+    return a.defer_reduce ? launch_mid_reduce(c.rg, c.mt, wn, a, stream) : SG_SUCCESS;
 }
 
 // Mid-batch heuristic, fitted to timings of the Llama-3-70B projection shapes at M = 64..256:
@@ -530,7 +580,10 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     c.engine = ENGINE_MID;
     c.nt = 1;
     c.persist = 0;
-    c.wavetile = 0;
+    // a K split leaves its sum to a second launch over the whole device: level or ahead of the last workgroup's serial
+    // sum on every split record of the Llama-3-70B shapes (128 x 128 tiles split three ways at 128 x 10240 x 8192
+    // 32.1 -> 26.6 us, 128 x 64 split four ways at 64 x 8192 x 28672 46.8 -> 43.6, 64 x 64 split in two 19.1 -> 18.5)
+    c.wavetile = c.split_k > 1 ? 1 : 0;
     const int bn = 8 * c.rg * c.waves, bm = 32 * c.mt;
     const int per_wave_w = bn / (8 * c.waves), per_wave_x = bm / (8 * c.waves);   // DMA instructions per wave and stage
     // (weight slots, activation slots; 0 = as many): the deepest ring that fits 160 KB.  A shallower
@@ -548,7 +601,7 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
             if (dw == 4 && dx == 3 && c.waves != 14) continue;   // compiled for the 224 x 128 tile, which it fills to 160 KB
             const int in_flight_x = per_wave_w + (dx - 2) * (per_wave_w + per_wave_x);
             const int in_flight_w = (dw - 2) * (per_wave_w + per_wave_x);
-            const size_t lds = ((size_t)dw * bn + (size_t)dx * bm) * 128 + (c.split_k > 1 ? 16 : 0);   // + arrival word
+            const size_t lds = ((size_t)dw * bn + (size_t)dx * bm) * 128;   // (a split's sum is a second launch: no arrival word)
             if (lds > 160 * 1024) continue;
             if ((in_flight_x < in_flight_w ? in_flight_x : in_flight_w) > 63) continue;
             c.depth = dw;
@@ -629,6 +682,27 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
         }
     }
     return c;
+}
+
+// Split-K partial bytes and arrival counters the launch of `c` on an m x n x k problem takes from its workspace
+// (zero without a K split): the arithmetic of prepare() / launch_mid_engine() without the launch.
+static void workspace_need(const Config& c, int m, int n, size_t* partial_bytes, size_t* counters) {
+    *partial_bytes = 0;
+    *counters = 0;
+    if (c.split_k <= 1) return;
+    size_t tiles, per_tile;
+    if (c.engine == ENGINE_MID) {
+        const int wn = c.waves / 2;
+        const int bn = 16 * c.rg * (wn > 0 ? wn : 1), bm = 32 * c.mt;
+        tiles = (size_t)((n + bn - 1) / bn) * ((m + bm - 1) / bm);
+        per_tile = (size_t)c.waves * c.rg * c.mt * 1024;
+    } else {
+        const int tile_rows = (c.engine == ENGINE_LDS && (c.wavetile & 8)) ? 24 : 16 * c.rg;
+        tiles = (size_t)((n + tile_rows - 1) / tile_rows) * ((m + 16 * c.mt - 1) / (16 * c.mt));
+        per_tile = (size_t)c.rg * c.mt * 1024;
+    }
+    *partial_bytes = tiles * c.split_k * per_tile;
+    *counters = tiles;
 }
 
 static int launch_config(const Config& c, const StreamArgs& a, hipStream_t stream) {
@@ -942,6 +1016,7 @@ static int get_act_scratch(hipStream_t stream, size_t bytes, uint8_t** out) {
         const size_t want = round_up_pow2(bytes, 1u << 20);
         void* p = workspace_alloc(want);    // an outgrown buffer is kept: launches already enqueued may still read it
         if (!p) return SG_NO_DEVICE;
+        if (sc.p) g_retired[dev].push_back({stream, sc.p, sc.bytes});
         sc.p = static_cast<uint8_t*>(p);
         sc.bytes = want;
         g_ws_bytes[dev] += want;
@@ -1046,8 +1121,34 @@ static Config heuristic_config(int m, int n, int k, int cu_count) {
 static std::mutex g_table_mutex;
 static std::map<std::tuple<int, int, int>, SgTuning> g_table;
 static std::atomic<int> g_table_entries{0};   // an empty table costs the launch path one relaxed load
+static int sg_tuning_load_file(const char* path);   // what sg_tuning_load does, without the default table first
+
+// The table the library ships: tuning/mi355x.tbl beside the package's csrc directory (the records its tuning driver
+// found for the benchmark shapes), merged into the table once, before the table is first read or changed.  The
+// environment variable SGEMM_TUNING_TABLE names another file to load instead; empty or "none" loads nothing.
+static std::once_flag g_default_table_once;
+static void load_default_table() {
+    const char* env = std::getenv("SGEMM_TUNING_TABLE");
+    if (env) {
+        if (*env && std::strcmp(env, "none") != 0 && sg_tuning_load_file(env) != SG_SUCCESS && std::getenv("SG_VERBOSE"))
+            std::fprintf(stderr, "libsgemm: cannot load the tuning table %s\n", env);
+        return;
+    }
+    Dl_info info;
+    if (!dladdr(reinterpret_cast<const void*>(&load_default_table), &info) || !info.dli_fname) return;
+    std::string path(info.dli_fname);
+    const size_t slash = path.rfind('/');
+    path = (slash == std::string::npos ? std::string(".") : path.substr(0, slash)) + "/../tuning/mi355x.tbl";
+    if (FILE* f = std::fopen(path.c_str(), "r")) {
+        std::fclose(f);
+        if (sg_tuning_load_file(path.c_str()) != SG_SUCCESS && std::getenv("SG_VERBOSE"))
+            std::fprintf(stderr, "libsgemm: malformed tuning table %s\n", path.c_str());
+    }
+}
+static void ensure_default_table() { std::call_once(g_default_table_once, load_default_table); }
 
 static bool table_lookup(int m, int n, int k, SgTuning* out) {
+    ensure_default_table();
     if (g_table_entries.load(std::memory_order_relaxed) == 0) return false;
     std::lock_guard<std::mutex> lock(g_table_mutex);
     const auto it = g_table.find(std::make_tuple(m, n, k));
@@ -1133,11 +1234,119 @@ size_t sg_workspace_bytes(void) {
     return g_ws_bytes[dev];
 }
 
+// Frees the buffers of g_ws / g_act / g_retired that belong to `stream` (all streams with every == true); the caller
+// has synchronised.  g_mutex held.
+static void free_owned(int dev, hipStream_t stream, bool every) {
+    for (auto it = g_ws[dev].begin(); it != g_ws[dev].end();) {
+        if (every || it->first == stream) {
+            if (it->second.partials) { (void)hipFree(it->second.partials); g_ws_bytes[dev] -= it->second.partial_bytes; }
+            if (it->second.counters) { (void)hipFree(it->second.counters); g_ws_bytes[dev] -= it->second.n_counters * sizeof(unsigned); }
+            it = g_ws[dev].erase(it);
+        } else {
+            ++it;
+        }
+    }
+    for (auto it = g_act[dev].begin(); it != g_act[dev].end();) {
+        if (every || it->first == stream) {
+            if (it->second.p) { (void)hipFree(it->second.p); g_ws_bytes[dev] -= it->second.bytes; }
+            it = g_act[dev].erase(it);
+        } else {
+            ++it;
+        }
+    }
+    std::vector<Retired> keep;
+    for (const Retired& r : g_retired[dev]) {
+        if (every || r.stream == stream) { (void)hipFree(r.p); g_ws_bytes[dev] -= r.bytes; }
+        else keep.push_back(r);
+    }
+    g_retired[dev].swap(keep);
+}
+
+int sg_release_stream(void* stream) {
+    int dev;
+    if (int rc = current_device(&dev)) return rc;
+    if (report_hip("hipStreamSynchronize", hipStreamSynchronize(static_cast<hipStream_t>(stream))) != hipSuccess) {
+        (void)hipGetLastError();
+        return SG_LAUNCH_FAILED;
+    }
+    std::lock_guard<std::mutex> lock(g_mutex);
+    free_owned(dev, static_cast<hipStream_t>(stream), false);
+    return SG_SUCCESS;
+}
+
+int sg_release_workspaces(void) {
+    int dev;
+    if (int rc = current_device(&dev)) return rc;
+    if (report_hip("hipDeviceSynchronize", hipDeviceSynchronize()) != hipSuccess) {
+        (void)hipGetLastError();
+        return SG_LAUNCH_FAILED;
+    }
+    std::lock_guard<std::mutex> lock(g_mutex);
+    free_owned(dev, nullptr, true);
+    return SG_SUCCESS;
+}
+
+// Caller-owned workspace: [kCallerCounters arrival counters][fp32 partials].  The counter region has one size for
+// every shape, so that one buffer serves launches of different shapes one after the other.
+constexpr size_t kCallerCounters = 16384;
+constexpr size_t kCallerCounterBytes = kCallerCounters * sizeof(unsigned);
+
+int sg_workspace_query(int m, int n, int k, size_t* bytes) {
+    if (!bytes || m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    int cu = 256;
+    if (get_device_info(&dev) == SG_SUCCESS) cu = dev->cu_count;
+    SgTuning t;
+    Config c = (table_lookup(m, n, k, &t) && t.engine != ENGINE_AUTO) ? config_from_tuning(t) : heuristic_config(m, n, k, cu);
+    size_t partial, counters;
+    workspace_need(c, m, n, &partial, &counters);
+    // (should the table's record be refused at launch, the heuristics' record runs: it must fit as well)
+    const Config h = heuristic_config(m, n, k, cu);
+    size_t partial_h, counters_h;
+    workspace_need(h, m, n, &partial_h, &counters_h);
+    if (partial_h > partial) partial = partial_h;
+    *bytes = partial ? kCallerCounterBytes + partial : 0;
+    return SG_SUCCESS;
+}
+
+int sg_workspace_init(void* workspace, size_t bytes, void* stream) {
+    if (!workspace || bytes < kCallerCounterBytes || (reinterpret_cast<uintptr_t>(workspace) & 255u)) return SG_BAD_ARGUMENT;
+    return fill_zero(static_cast<unsigned*>(workspace), kCallerCounters, static_cast<hipStream_t>(stream));
+}
+
+int sg_skinny_gemm_auto_ws(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,
+                           int b_stride, void* workspace, size_t workspace_bytes, void* stream) {
+    if (n % 2 != 0) return SG_N_NOT_EVEN;
+    if (k % 16 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (int rc = check_pointers(A, B, D, m, n, k, b_stride)) return rc;
+    if (!scale_tensor) return SG_BAD_ARGUMENT;
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u)) return SG_BAD_ALIGNMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    size_t need = 0;
+    if (int rc = sg_workspace_query(m, n, k, &need)) return rc;
+    if (need > 0 && (!workspace || workspace_bytes < need)) return SG_WORKSPACE_TOO_SMALL;
+    // a launch without a K split gets a workspace nothing fits into: whatever would want one is refused, never allocated
+    Workspace w;
+    if (need > 0) {
+        w.counters = static_cast<unsigned*>(workspace);
+        w.n_counters = kCallerCounters;
+        w.partials = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + kCallerCounterBytes);
+        w.partial_bytes = workspace_bytes - kCallerCounterBytes;
+    }
+    StreamArgs a{};
+    a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
+    a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
+    a.out_f32 = 0;
+    return launch_chosen(a, dev->cu_count, static_cast<hipStream_t>(stream), &w);
+}
+
 int sg_debug_stamps(unsigned long long* device_buffer, size_t n_words) {
     std::lock_guard<std::mutex> lock(g_mutex);
     g_stamp_buf = n_words ? device_buffer : nullptr;
     g_stamp_words = device_buffer ? n_words : 0;
     g_stamp_cursor = 0;
+    g_stamps_on.store(g_stamp_buf != nullptr && g_stamp_words > 0, std::memory_order_relaxed);
     return SG_SUCCESS;
 }
 
@@ -1247,7 +1456,8 @@ int sg_skinny_gemm_tuned_noalloc(const uint8_t* A, const uint8_t* B, void* D, co
     DeviceInfo* dev;
     if (int rc = get_device_info(&dev)) return rc;
     Workspace w;
-    if (int rc = static_workspace(&w)) return rc;
+    bool first_use = false;
+    if (int rc = static_workspace(&w, &first_use)) return rc;
     Config c = config_from_tuning(*t);
     if (c.engine == ENGINE_AUTO) c = heuristic_config(m, n, k, dev->cu_count);
     if (c.engine != ENGINE_MID && c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
@@ -1256,11 +1466,12 @@ int sg_skinny_gemm_tuned_noalloc(const uint8_t* A, const uint8_t* B, void* D, co
     a.A = A; a.B = B; a.D = D; a.scale = scale_tensor;
     a.m = m; a.n = n; a.k = k; a.b_stride = b_stride;
     a.out_f32 = 0;
-    // The array keeps whatever the last call left.  The partials are written before they are read; the arrival
-    // counters must start at zero, and although a launch that completes leaves them at zero they are cleared
-    // here, in stream order, with a kernel (a memset node would not be safe in a captured graph).
-    if (c.split_k > 1)
-        if (int rc = fill_zero(w.counters, w.n_counters, static_cast<hipStream_t>(stream))) return rc;
+    // The array keeps whatever the last call left.  The partials are written before they are read.  The arrival
+    // counters must start at zero: the array is zero when the device image is loaded and every launch that completes
+    // leaves its counters at zero, so they are cleared once, with the first call on the device (by a kernel, at once:
+    // under capture a launch on the stream would only be recorded), and not again before every launch.
+    if (first_use)
+        if (int rc = fill_zero_now(w.counters, w.n_counters)) return rc;
     return launch_config(c, a, static_cast<hipStream_t>(stream));
 }
 
@@ -1409,6 +1620,7 @@ int sg_skinny_gemm_bf16act_choice(int m, int n, int k, SgTuning* out, int* fused
 
 int sg_tuning_set(int m, int n, int k, const SgTuning* t) {
     if (m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
+    ensure_default_table();
     std::lock_guard<std::mutex> lock(g_table_mutex);
     if (t) {
         if (t->engine != ENGINE_DIRECT && t->engine != ENGINE_LDS && t->engine != ENGINE_MID) return SG_INVALID_CONFIG;
@@ -1425,9 +1637,13 @@ int sg_tuning_get(int m, int n, int k, SgTuning* out) {
     return table_lookup(m, n, k, out) ? SG_SUCCESS : SG_INVALID_CONFIG;
 }
 
-int sg_tuning_count(void) { return g_table_entries.load(std::memory_order_relaxed); }
+int sg_tuning_count(void) {
+    ensure_default_table();
+    return g_table_entries.load(std::memory_order_relaxed);
+}
 
 int sg_tuning_clear(void) {
+    ensure_default_table();
     std::lock_guard<std::mutex> lock(g_table_mutex);
     g_table.clear();
     g_table_entries.store(0, std::memory_order_relaxed);
@@ -1438,6 +1654,14 @@ int sg_tuning_clear(void) {
 //   m n k engine split_k waves row_tiles m_blocks depth k_chunks non_temporal persistent_wgs_per_cu wave_tiles
 // '#' starts a comment; blank lines are skipped.
 int sg_tuning_load(const char* path) {
+    ensure_default_table();
+    return sg_tuning_load_file(path);
+}
+
+}  // extern "C"
+
+namespace sg {
+static int sg_tuning_load_file(const char* path) {
     if (!path) return SG_BAD_ARGUMENT;
     FILE* f = std::fopen(path, "r");
     if (!f) return SG_BAD_ARGUMENT;
@@ -1478,9 +1702,13 @@ int sg_tuning_load(const char* path) {
     g_table_entries.store((int)g_table.size(), std::memory_order_relaxed);
     return SG_SUCCESS;
 }
+}  // namespace sg
+
+extern "C" {
 
 int sg_tuning_save(const char* path) {
     if (!path) return SG_BAD_ARGUMENT;
+    ensure_default_table();
     FILE* f = std::fopen(path, "w");
     if (!f) return SG_BAD_ARGUMENT;
     std::fprintf(f, "sgemm-tuning 1\n# m n k engine split_k waves row_tiles m_blocks depth k_chunks non_temporal "

@@ -36,6 +36,7 @@ struct StreamArgs {
     unsigned inv_n_tiles, inv_split_k, inv_waves;  // div_reciprocal() of n_tiles, split_k, waves (set_reciprocals)
     unsigned long long* stamps;  // profiling aid, normally nullptr: kStampWords time stamps per workgroup (sg_debug_stamps)
     int x_extra;            // register-resident kernel: 1 = the launch's LDS has one more 4 KB staging block per wave behind the reduction scratch
+    int defer_reduce;       // mid-batch kernel with split_k > 1: 1 = store the fp32 partials only; a second launch (mid_reduce_kernel) sums them
 };
 
 // Time stamps a workgroup leaves when a.stamps is set (wave 0 writes them when it is done):

@@ -45,6 +45,8 @@ int SG_RING_LAUNCHER(2)(int bl, int xu, int nt, const RingArgs& ra, unsigned gri
 int launch_xreg(int mt, int rg, int pt, int depth, const StreamArgs& a, unsigned grid, unsigned threads, size_t lds,
                 hipStream_t stream);
 int launch_mid(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream);
+// second launch of a mid-batch GEMM with StreamArgs::defer_reduce: sums the split-K partials of every output fragment
+int launch_mid_reduce(int rgw, int mh, int wn, const StreamArgs& a, hipStream_t stream);
 
 struct SparseArgs;
 int launch_sparse(int mt, int rg, int xu2, int depth, const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds,

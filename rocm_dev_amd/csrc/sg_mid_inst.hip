@@ -51,6 +51,13 @@ static int launch_mid_tail(int rgw, int mh, int depth, int dx, int wn, const Str
     return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
 }
 
+int launch_mid_reduce(int rgw, int mh, int wn, const StreamArgs& a, hipStream_t stream) {
+    const size_t items = (size_t)a.n_tiles * a.m_tiles * 2 * wn * rgw * mh;   // one wave each, four to a workgroup
+    if (items == 0 || (items + 3) / 4 > 0x7fffffffu) return SG_BAD_ARGUMENT;
+    mid_reduce_kernel<<<dim3((unsigned)((items + 3) / 4)), dim3(256), 0, stream>>>(a, rgw, mh, wn);
+    return report_hip("mid_reduce_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
+}
+
 int launch_mid(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, unsigned grid, size_t lds, hipStream_t stream) {
     if (a.k & 127) return launch_mid_tail(rgw, mh, depth, dx, wn, a, grid, lds, stream);
     SG_CASE_7(8, 3, 2) SG_CASE_7(8, 2, 2)                                       // 224 x 256: 84 + 64 KB

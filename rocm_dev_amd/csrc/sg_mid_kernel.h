@@ -25,6 +25,10 @@
 //
 // K is split across workgroups when there are few tiles; partials meet in the fp32 workspace
 // and the last workgroup to arrive sums them in split order (same scheme as the skinny path).
+// With large tiles that sum is a long serial tail in one workgroup (a 256 x 128 tile split four ways:
+// 512 KB read back by one CU while the others have left), so a launch may instead store its partials
+// only (StreamArgs::defer_reduce) and leave the sum to mid_reduce_kernel, a second launch that spreads
+// it over the whole device, one wave per 16 x 16 fragment; same split order, same result bits.
 // Inside its K range a workgroup starts at a block that depends on its weight tile and wraps
 // around, so the fp32 sum of an output element is taken in a rotated - still fixed - K order.
 #pragma once
@@ -312,6 +316,15 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     constexpr int FRAGS_WG = WAVES * RGW * MH;   // fragments of one workgroup tile
     const int tile_id = tile_m * a.n_tiles + tile_n;
     float* ws_tile = a.ws + ((size_t)tile_id * a.split_k) * (FRAGS_WG * 256);
+    if (a.defer_reduce) {
+        // partials only: [tile][split][wave][fragment][lane] as one 16-byte store per lane and fragment
+        f32x4* mine = reinterpret_cast<f32x4*>(ws_tile + (size_t)split * (FRAGS_WG * 256) + (size_t)wave * (RGW * MH * 256)) + lane;
+#pragma unroll
+        for (int rg = 0; rg < RGW; rg++)
+#pragma unroll
+            for (int mb = 0; mb < MH; mb++) mine[(rg * MH + mb) * 64] = acc[rg][mb];
+        return;
+    }
     {
         float* mine = ws_tile + (size_t)split * (FRAGS_WG * 256) + (size_t)wave * (RGW * MH * 256) + lane;
 #pragma unroll
@@ -341,6 +354,30 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         return v;
     });
     if (threadIdx.x == 0) __hip_atomic_store(&a.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+
+// Second launch of a mid-batch GEMM whose split-K sum was deferred: one wave per 16 x 16 fragment of the output adds
+// the fragment's split_k partials in split order - what the last workgroup to arrive does in the single launch, so
+// the result bits are the same - and applies scale, row and column factors and the rounding.  The tile geometry
+// comes as run-time values: rgw x mh fragments per wave, wn x 2 waves per tile.
+__global__ void __launch_bounds__(256) mid_reduce_kernel(const StreamArgs a, int rgw, int mh, int wn) {
+    const int fr = rgw * mh, frags_wg = 2 * wn * fr;
+    const int lane = lane_id();
+    const unsigned item = blockIdx.x * 4u + (unsigned)wave_id();      // (tile, wave of the tile, fragment of the wave)
+    const unsigned tile_id = item / (unsigned)frags_wg, rem = item - tile_id * (unsigned)frags_wg;
+    if (tile_id >= (unsigned)(a.n_tiles * a.m_tiles)) return;
+    const int wave = (int)rem / fr, f = (int)rem - wave * fr;
+    const int rg = f / mh, mb = f - rg * mh;
+    const int tile_m = (int)tile_id / a.n_tiles, tile_n = (int)tile_id - tile_m * a.n_tiles;
+    const int wq = wave % wn, wm = wave / wn;
+    const f32x4* p = reinterpret_cast<const f32x4*>(a.ws + ((size_t)tile_id * a.split_k) * ((size_t)frags_wg * 256) +
+                                                    (size_t)wave * (fr * 256) + (size_t)f * 256) + lane;
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < a.split_k; sp++) v += p[(size_t)sp * ((size_t)frags_wg * 64)];
+    const float scale = a.scale ? a.scale[0] : 1.0f;
+    const int r = lane & 15, g = lane >> 4;
+    store_fragment(a, v, scale, tile_m * (32 * mh) + (wm * mh + mb) * 16 + r, tile_n * (16 * rgw * wn) + (wq * rgw + rg) * 16 + 4 * g);
 }
 
 }  // namespace sg

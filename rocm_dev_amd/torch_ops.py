@@ -26,10 +26,22 @@ def _bytes(t):
     return t.view(torch.uint8) if t.dtype == torch.float8_e4m3fn else t
 
 
+def _rows(t):
+    """Activations and vectors in the row-major layout the kernels read: eager code and torch.compile may hand a
+    functional operator a transposed or sliced view, which is copied here (a no-op for contiguous tensors)."""
+    return None if t is None else _bytes(t).contiguous()
+
+
+def _weights(t):
+    """Weights stay where they are - [n, k] with k contiguous, rows at any stride of at least k; anything else is
+    refused by the api layer rather than copied (a silent copy of a weight matrix per call is a bug in the caller)."""
+    return _bytes(t)
+
+
 @torch.library.custom_op("sgemm::skinny_gemm", mutates_args=())
 def skinny_gemm(A: torch.Tensor, B: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     D = torch.empty((A.shape[0], B.shape[0]), dtype=torch.bfloat16, device=A.device)
-    api.skinny_gemm_fastpath(_bytes(A), _bytes(B), D, scale, check=True)
+    api.skinny_gemm_fastpath(_rows(A), _weights(B), D, _rows(scale), check=True)
     return D
 
 
@@ -42,7 +54,7 @@ def _(A, B, scale):
 def skinny_gemm_rowcol(A: torch.Tensor, B: torch.Tensor, scale: Optional[torch.Tensor] = None,
                        row_scales: Optional[torch.Tensor] = None, col_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
     D = torch.empty((A.shape[0], B.shape[0]), dtype=torch.bfloat16, device=A.device)
-    api.skinny_gemm_rowcol(_bytes(A), _bytes(B), D, scale, row_scales, col_scales, check=True)
+    api.skinny_gemm_rowcol(_rows(A), _weights(B), D, _rows(scale), _rows(row_scales), _rows(col_scales), check=True)
     return D
 
 
@@ -55,7 +67,7 @@ def _(A, B, scale=None, row_scales=None, col_scales=None):
 def skinny_gemm_bf16act(X: torch.Tensor, B: torch.Tensor, scale: Optional[torch.Tensor] = None,
                         col_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
     D = torch.empty((X.shape[0], B.shape[0]), dtype=torch.bfloat16, device=X.device)
-    api.skinny_gemm_bf16act(X, _bytes(B), D, scale, col_scales, check=True)
+    api.skinny_gemm_bf16act(_rows(X), _weights(B), D, _rows(scale), _rows(col_scales), check=True)
     return D
 
 
@@ -68,7 +80,7 @@ def _(X, B, scale=None, col_scales=None):
 def fp8_encode_rows(X: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     Q = torch.empty(X.shape, dtype=torch.uint8, device=X.device)
     s = torch.empty((X.shape[0],), dtype=torch.float32, device=X.device)
-    api.fp8_encode_rows(X, Q, s, check=True)
+    api.fp8_encode_rows(_rows(X), Q, s, check=True)
     return Q, s
 
 
@@ -80,7 +92,7 @@ def _(X):
 @torch.library.custom_op("sgemm::fp8_decode_rows", mutates_args=())
 def fp8_decode_rows(Q: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
     Y = torch.empty(Q.shape, dtype=torch.bfloat16, device=Q.device)
-    api.fp8_decode_rows(_bytes(Q), scales, Y, check=True)
+    api.fp8_decode_rows(_rows(Q), _rows(scales), Y, check=True)
     return Y
 
 
@@ -92,7 +104,7 @@ def _(Q, scales):
 @torch.library.custom_op("sgemm::sparse24_gemm", mutates_args=())
 def sparse24_gemm(A: torch.Tensor, vals: torch.Tensor, meta: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     D = torch.empty((A.shape[0], vals.shape[0]), dtype=torch.bfloat16, device=A.device)
-    api.sparse24_gemm(_bytes(A), vals, meta, D, scale, check=True)
+    api.sparse24_gemm(_rows(A), _rows(vals), _rows(meta), D, _rows(scale), check=True)
     return D
 
 

@@ -120,6 +120,9 @@ def expect_mid(m, n, k, r):
     32*m_blocks activation rows, `depth` weight slots and `k_chunks` (or depth) activation slots of
     128 bytes of K."""
     waves, rg, mt, depth, sk, dx = r["waves"], r["row_tiles"], r["m_blocks"], r["depth"], r["split_k"], r["k_chunks"]
+    wt = r.get("wave_tiles", 0)
+    # a split whose sum is a second launch (wave_tiles = 1) needs no arrival word in LDS
+    arrival = 16 if sk > 1 and wt != 1 else 0
     if k % 128:
         # a partial last block: only beyond 128, and only in the builds listed below
         if k % 16 or k <= 128:
@@ -128,9 +131,11 @@ def expect_mid(m, n, k, r):
             return INVALID
         if not 1 <= sk <= k // 128:
             return INVALID
+        if wt not in (0, 1):
+            return INVALID
         d = dx if 2 <= dx < depth else depth
         wn_ = waves // 2
-        if (depth * 16 * rg * wn_ + d * 32 * mt) * 128 + (16 if sk > 1 else 0) > 160 * 1024:
+        if (depth * 16 * rg * wn_ + d * 32 * mt) * 128 + arrival > 160 * 1024:
             return INVALID
         return OK if (rg, mt, depth, wn_, d) in _MID_TAIL else 3
     if rg not in (2, 4) or mt not in (2, 4, 8) or depth < 2 or waves not in (4, 8, 14):
@@ -141,8 +146,10 @@ def expect_mid(m, n, k, r):
         return INVALID
     if not 1 <= sk <= k // 128:
         return INVALID
+    if wt not in (0, 1):
+        return INVALID
     dx = dx if 2 <= dx < depth else depth
-    if (depth * bn + dx * bm) * 128 + (16 if sk > 1 else 0) > 160 * 1024:
+    if (depth * bn + dx * bm) * 128 + arrival > 160 * 1024:
         return INVALID
     if wn == 7:
         return OK if (rg, mt, depth, dx) in _MID_7 else INVALID

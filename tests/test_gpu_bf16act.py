@@ -114,7 +114,7 @@ def test_decode_shapes_fused_kernel(sg, oracle, m, n, k):
         B = torch.zeros((n, k), dtype=torch.uint8, device="cuda")
         D = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
         assert sg.skinny_gemm_bf16act(X, B, D, tuning=sg.SgTuning()) == 6
-        pytest.skip("the activation codes do not fit LDS beside four waves' rings, and the library says so")
+        return   # the refusal asserted above is this case\'s expected result (the activation codes do not fit LDS beside four waves' rings, and the library says so)
     _both_ways(sg, oracle, m, n, k, seed=m, force=True)
 
 

@@ -103,7 +103,7 @@ def test_sparse_tuned_configs(sg, oracle, cfg, shape):
     want = expect_sparse(m, n, k, record(2, split_k, waves, row_tiles, 1 if m <= 16 else 2, depth))
     assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
     if rc != 0:
-        pytest.skip("the configuration does not fit this shape, and the library says so")
+        return   # the refusal asserted above is this case\'s expected result (the configuration does not fit this shape, and the library says so)
     assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
     rc, again = _run(sg, a8, vals, meta, scale, tuning=t)
     assert rc == 0 and np.array_equal(again, got)
@@ -135,7 +135,7 @@ def test_sparse_wave_per_tile_configs(sg, oracle, cfg, shape):
     want = expect_sparse(m, n, k, record(2, 1, waves, row_tiles, 1, depth, 8, 1, per_cu, 1))
     assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
     if rc != 0:
-        pytest.skip("the configuration does not fit this shape, and the library says so")
+        return   # the refusal asserted above is this case\'s expected result (the configuration does not fit this shape, and the library says so)
     assert oracle.max_rel_err_bf16(got, ref) <= GEMM_TOL
     rc, again = _run(sg, a8, vals, meta, scale, tuning=t)
     assert rc == 0 and np.array_equal(again, got)

@@ -110,3 +110,42 @@ def test_driver_measures_checks_and_writes_a_loadable_table(sg, oracle, tmp_path
     sg.tuning_load(out)
     assert sg.tuning_count() == 2
     assert oracle.max_rel_err_bf16(_fast(sg, A, B, S, m, n), ref) <= GEMM_TOL
+
+
+def test_the_shipped_table_against_the_oracle(sg, oracle):
+    """Every record of rocm_dev_amd/tuning/mi355x.tbl at its own shape, through the fastpath with the table loaded
+    the way a user's process loads it: two 256-row slices of the output against the CPU oracle."""
+    import os
+
+    import numpy as np
+    import torch
+
+    from gpu_util import GEMM_TOL, bits, dev, gemm_reference, scale_tensor
+    from rocm_dev_amd import api, autotune
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "rocm_dev_amd", "tuning", "mi355x.tbl")
+    entries = autotune.parse_table(open(path).read())
+    sg.tuning_clear()
+    sg.tuning_load(path)
+    try:
+        for (m, n, k), r in sorted(entries.items()):
+            choice, from_table = sg.skinny_gemm_choice(m, n, k)
+            assert from_table and api.tuning_as_dict(choice) == r
+            a = oracle.normal_f32((m, k), 0, 1)
+            a8, sa = oracle.quantize_tensor(a)
+            g = torch.Generator(device="cuda").manual_seed(m + n)
+            w = torch.randn((n, k), generator=g, device="cuda", dtype=torch.float32)
+            sb = w.abs().max() / 448.0
+            B = (w / sb).to(torch.float8_e4m3fn).view(torch.uint8)
+            del w
+            scale = np.float32(sa) * np.float32(sb.item())
+            D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+            assert sg.skinny_gemm_fastpath(dev(a8), B, D, scale_tensor(scale)) == 0
+            torch.cuda.synchronize()
+            got = bits(D)
+            assert not np.isnan(oracle.bf16_to_f32(got)).any(), (m, n, k)
+            for lo in (0, n - 256):
+                ref = gemm_reference(oracle, a8, B[lo:lo + 256].cpu().numpy(), scale)
+                assert oracle.max_rel_err_bf16(got[:, lo:lo + 256], ref) <= GEMM_TOL, (m, n, k, lo)
+            del B, D
+    finally:
+        sg.tuning_clear()

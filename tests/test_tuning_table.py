@@ -251,3 +251,42 @@ def test_the_heuristics_only_choose_what_the_launchers_take():
         choice, _ = sg.skinny_gemm_choice(m, n, k)
         assert choice.engine == engine and (engine != 2 or choice.wave_tiles == 1 or
                                             (choice.persistent_wgs_per_cu == 0 and choice.wave_tiles & 7 == 0)), (m, n, k)
+
+
+SHIPPED = __import__("os").path.join(__import__("os").path.dirname(__import__("os").path.dirname(__import__("os").path.abspath(__file__))),
+                                     "rocm_dev_amd", "tuning", "mi355x.tbl")
+
+
+def test_the_shipped_table_holds_launchable_records_for_benchmark_shapes():
+    """rocm_dev_amd/tuning/mi355x.tbl - what the tuning driver found on the benchmark shapes, the counterpart of the
+    reference committing its search result (skinny_gemm/core.cu:29-38): every record is one the launchers take
+    (the kernels' resource rules, restated independently in tests/launch_rules.py) for a shape of the presets."""
+    import launch_rules
+    entries = autotune.parse_table(open(SHIPPED).read())
+    assert entries, "an empty table would not need shipping"
+    shapes = set(autotune.PRESETS["baseline"])
+    for (m, n, k), r in entries.items():
+        assert (m, n, k) in shapes, (m, n, k)
+        expect = {1: None, 2: launch_rules.expect_lds, 4: launch_rules.expect_mid}[r["engine"]]
+        assert expect is not None and expect(m, n, k, r) == launch_rules.OK, (m, n, k, r)
+
+
+def test_the_shipped_table_is_loaded_once_unless_the_environment_says_otherwise(tmp_path):
+    """Loaded before the table is first read or changed; SGEMM_TUNING_TABLE names another file, "none" nothing."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    n_shipped = len(autotune.parse_table(open(SHIPPED).read()))
+    other = tmp_path / "other.tbl"
+    other.write_text(autotune.format_table({(8, 4096, 4096): autotune.record(2, 1, 3, 1, 1, 4)}.items()))
+    code = ("import rocm_dev_amd as sg; print(sg.tuning_count()); "
+            "t = sg.tuning_get(128, 10240, 8192); print(-1 if t is None else t.split_k); "
+            "sg.tuning_clear(); print(sg.tuning_count())")
+    for value, want in ((None, [n_shipped, 3, 0]), ("none", [0, -1, 0]), ("", [0, -1, 0]), (str(other), [1, -1, 0])):
+        env = dict(os.environ)
+        env.pop("SGEMM_TUNING_TABLE", None)
+        if value is not None:
+            env["SGEMM_TUNING_TABLE"] = value
+        out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, check=True)
+        assert [int(v) for v in out.stdout.split()] == want, (value, out.stdout, out.stderr)
