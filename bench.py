@@ -281,16 +281,23 @@ def main():
 
     if args.stamps:
         import numpy as np
+        from rocm_dev_amd import synth as _synth
+        quantize = _synth.quantize_tensor       # N(0,1) operands quantised per tensor, as in the timed runs
         one = torch.ones(1, device="cuda")
         reps = 24
         print("in-kernel time stamps, M = %d, graph of %d back-to-back launches on cold weights, medians over launches 4..%d"
               % (args.m, reps, reps - 1))
         print("all times in us; gap = first entry of a launch - last end of the one before; spread = last - first entry")
         side = torch.cuda.Stream()
-        for name, (n, k) in SHAPES.items():
+        # the four decode projections at --m, or the shapes of --launch-shapes MxNxK (each with its own M)
+        jobs = [(name, args.m, n, k) for name, (n, k) in SHAPES.items()]
+        if args.launch_shapes:
+            jobs = [(s, *[int(v) for v in s.lower().split("x")]) for s in args.launch_shapes]
+        for name, m_, n, k in jobs:
+            args.m = m_
             copies = max(3, int(COLD_BYTES // (n * k)) + 1)
-            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(copies)]
-            a8 = torch.randint(0, 0x7E, (args.m, k), device="cuda", dtype=torch.uint8)
+            wb = [quantize(torch.randn((n, k), device="cuda", dtype=torch.float32))[0] for _ in range(copies)]
+            a8 = quantize(torch.randn((args.m, k), device="cuda", dtype=torch.float32))[0]
             d = torch.empty((args.m, n), device="cuda", dtype=torch.bfloat16)
             words = reps * 4096 * 8
             buf = torch.zeros(words, device="cuda", dtype=torch.int64)
@@ -332,7 +339,7 @@ def main():
                     "mhz": np.median((t[j, :, 6].astype(np.int64) - t[j, :, 5].astype(np.int64)) / np.maximum(end[j] - ent[j], tick))})
             med = {key: float(np.median([r[key] for r in rows])) for key in rows[0]}
             t_choice, _ = sg.skinny_gemm_choice(args.m, n, k)
-            print("%-8s %5d x %5d  grid %4d  event-pair period %.2f | period %.2f = gap %.2f + span %.2f | entry spread %.2f | "
+            print("%-18s %5d x %5d  grid %4d  event-pair period %.2f | period %.2f = gap %.2f + span %.2f | entry spread %.2f | "
                   "workgroup (median): prologue issue %.2f, first stage landed %.2f (max %.2f), streaming %.2f, reduce+store %.2f, "
                   "total %.2f (max %.2f) | last end - median end %.2f | shader clock %.0f MHz | %s"
                   % (name, n, k, grid, period_ev, med["period"], med["gap"], med["span"], med["spread"], med["issue"], med["land_med"],

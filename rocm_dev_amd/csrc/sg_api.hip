@@ -491,6 +491,7 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
     a.defer_reduce = (c.wavetile == 1 && c.split_k > 1) ? 1 : 0;
     const size_t lds = ((size_t)c.depth * bn + (size_t)dx * bm) * 128 + ((c.split_k > 1 && !a.defer_reduce) ? 16 : 0);
     if (lds > 160 * 1024) return SG_INVALID_CONFIG;
+    a.stamps = take_stamps((unsigned)(tiles * c.split_k));
     if (int rc = launch_mid(c.rg, c.mt, c.depth, dx, wn, a, (unsigned)(tiles * c.split_k), lds, stream)) return rc;
     return a.defer_reduce ? launch_mid_reduce(c.rg, c.mt, wn, a, stream) : SG_SUCCESS;
 }

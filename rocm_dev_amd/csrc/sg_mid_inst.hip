@@ -52,9 +52,11 @@ static int launch_mid_tail(int rgw, int mh, int depth, int dx, int wn, const Str
 }
 
 int launch_mid_reduce(int rgw, int mh, int wn, const StreamArgs& a, hipStream_t stream) {
-    const size_t items = (size_t)a.n_tiles * a.m_tiles * 2 * wn * rgw * mh;   // one wave each, four to a workgroup
-    if (items == 0 || (items + 3) / 4 > 0x7fffffffu) return SG_BAD_ARGUMENT;
-    mid_reduce_kernel<<<dim3((unsigned)((items + 3) / 4)), dim3(256), 0, stream>>>(a, rgw, mh, wn);
+    const int frags_wg = 2 * wn * rgw * mh;                    // fragments of a tile; a workgroup of four waves takes 4 * kReduceFrags
+    if ((rgw * mh) % kReduceFrags != 0) return SG_INVALID_CONFIG;
+    const size_t grid = (size_t)a.n_tiles * a.m_tiles * ((frags_wg + 4 * kReduceFrags - 1) / (4 * kReduceFrags));
+    if (grid == 0 || grid > 0x7fffffffu) return SG_BAD_ARGUMENT;
+    mid_reduce_kernel<<<dim3((unsigned)grid), dim3(256), 0, stream>>>(a, rgw, mh, wn);
     return report_hip("mid_reduce_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }
 

@@ -58,11 +58,36 @@ constexpr int mid_activation_waves(int instr, int waves) {
 //      from k - 128 - a window that ends with the row, nothing past it is read - and the activation fragments of that
 //      stage are zero in the 16-byte pieces the block before has already multiplied: lane (r, g) holds pieces g and
 //      g + 4 of a row, so that is a per-lane select.  (A build of its own: the loop for whole blocks stays as it is.)
+// Workgroup `bid` of a grid of `grid` -> the weight tile it works on and its position p (0 .. per_tile-1) among the
+// per_tile workgroups of that tile, in the order described in the kernel below: the weight tiles of XCD 0 (tile_n = 0,
+// 8, 16 ...) with all their workgroups, then XCD 1's, XCD x starting where its share of the grid starts.  Both
+// launches of a GEMM with a deferred split-K sum use it, so that the workgroups that sum a tile's partials run on the
+// XCD whose L2 the partials were last written through.
+__device__ __forceinline__ int xcd_weight_tile(int bid, int grid, int per_tile, int n_tiles, int& p) {
+    const int xcd = bid & 7, qs = grid >> 3, rs = grid & 7;
+    const int j = xcd * qs + (xcd < rs ? xcd : rs) + (bid >> 3);
+    const int r = j / per_tile;
+    p = j - r * per_tile;
+    const int qn = n_tiles >> 3, rn = n_tiles & 7;
+    int g, i;
+    if (r < rn * (qn + 1)) {
+        g = r / (qn + 1);
+        i = r - g * (qn + 1);
+    } else {                                 // (reached only with qn > 0: otherwise every r is below rn)
+        const int r2 = r - rn * (qn + 1);
+        g = rn + r2 / qn;
+        i = r2 - (g - rn) * qn;
+    }
+    return g + 8 * i;
+}
+
 template <int RGW, int MH, int DEPTH, int WN, int DX = DEPTH, bool TAIL = false>
 __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) {
     // [DEPTH][W rows][128] | [DX][X rows][128], then (split-K only) 16 bytes for the arrival broadcast; no
     // static LDS, so that two workgroups of exactly half the CU's LDS can share a CU
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
+    Stamps stamps;      // profiling aid: written out only when a.stamps is set (sg_debug_stamps)
+    stamps.begin();
 
     constexpr int WAVES = 2 * WN;
     constexpr int BN = 16 * RGW * WN;
@@ -98,22 +123,9 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     // share of the grid starts.  Tile counts that 8 does not divide put at most a few tiles on two XCDs.
     int tile_n, split, tile_m;
     {
-        const int bid = (int)blockIdx.x, grid = (int)gridDim.x;
-        const int xcd = bid & 7, qs = grid >> 3, rs = grid & 7;
-        const int j = xcd * qs + (xcd < rs ? xcd : rs) + (bid >> 3);
         const int per_tile = a.split_k * a.m_tiles;
-        const int r = j / per_tile, p = j - r * per_tile;
-        const int qn = a.n_tiles >> 3, rn = a.n_tiles & 7;
-        int g, i;
-        if (r < rn * (qn + 1)) {
-            g = r / (qn + 1);
-            i = r - g * (qn + 1);
-        } else {                                 // (reached only with qn > 0: otherwise every r is below rn)
-            const int r2 = r - rn * (qn + 1);
-            g = rn + r2 / qn;
-            i = r2 - (g - rn) * qn;
-        }
-        tile_n = g + 8 * i;
+        int p;
+        tile_n = xcd_weight_tile((int)blockIdx.x, (int)gridDim.x, per_tile, a.n_tiles, p);
         split = p / a.m_tiles;
         tile_m = p - split * a.m_tiles;
     }
@@ -284,6 +296,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         if (i < DX - 1 && i < n_blk) issue_x(i);
         if (i < n_blk) issue_w(i);
     }
+    stamps.mark(1);
     for (int s = 0; s < n_blk; s++) {
         // wait for this wave's part of stage s; everything issued after it may stay in flight.  Near the
         // end of the K range fewer stages follow, and the count is no longer known at compile time.
@@ -291,12 +304,15 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         else if (loads_x) wait_vmcnt<IN_FLIGHT>();
         else wait_vmcnt<IN_FLIGHT_W_ONLY>();
         __syncthreads();        // stage s is complete for every wave; stage s-1 has been consumed by every wave
+        if (s == 0) stamps.mark(2);
         __builtin_amdgcn_sched_barrier(0);
         // refills the slots of X(s-1) and W(s-1) on the way
         if constexpr (WN == 2) consume_burst(s, s + DX - 1, s + DEPTH - 1);
         else consume(s, s + DX - 1, s + DEPTH - 1);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
+
+    stamps.mark(3);
 
     // ---- epilogue --------------------------------------------------------------------------------
     const float scale = a.scale ? a.scale[0] : 1.0f;
@@ -309,6 +325,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     };
     if (a.split_k == 1) {
         store_all([&](int rg, int mb) { return acc[rg][mb]; });
+        stamps.end(a);
         return;
     }
 
@@ -323,6 +340,7 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         for (int rg = 0; rg < RGW; rg++)
 #pragma unroll
             for (int mb = 0; mb < MH; mb++) mine[(rg * MH + mb) * 64] = acc[rg][mb];
+        stamps.end(a);
         return;
     }
     {
@@ -342,7 +360,10 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
     if (threadIdx.x == 0)
         *arrival = __hip_atomic_fetch_add(&a.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    if (*arrival != (unsigned)(a.split_k - 1)) return;
+    if (*arrival != (unsigned)(a.split_k - 1)) {
+        stamps.end(a);
+        return;
+    }
     store_all([&](int rg, int mb) {
         const float* p = ws_tile + (size_t)wave * (RGW * MH * 256) + (rg * MH + mb) * 256 + lane;
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
@@ -354,30 +375,54 @@ __global__ void __launch_bounds__(WN * 128) mid_gemm_kernel(const StreamArgs a) 
         return v;
     });
     if (threadIdx.x == 0) __hip_atomic_store(&a.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    stamps.end(a);
 }
 
 
-// Second launch of a mid-batch GEMM whose split-K sum was deferred: one wave per 16 x 16 fragment of the output adds
-// the fragment's split_k partials in split order - what the last workgroup to arrive does in the single launch, so
-// the result bits are the same - and applies scale, row and column factors and the rounding.  The tile geometry
-// comes as run-time values: rgw x mh fragments per wave, wn x 2 waves per tile.
+// Second launch of a mid-batch GEMM whose split-K sum was deferred: every wave adds the split_k partials of
+// kReduceFrags 16 x 16 fragments of the output in split order - what the last workgroup to arrive does in the single
+// launch, so the result bits are the same - and applies scale, row and column factors and the rounding.  A wave's
+// work is a chain of round trips (partials, scale, store), so it takes several fragments at once and requests all
+// their partials of a split before it adds any: with one fragment per wave the launch took 7-12 us for 8-33 MB of
+// partials that the GEMM had just left in the caches.  The tile geometry comes as run-time values: rgw x mh
+// fragments per wave of the GEMM, wn x 2 waves per tile.
+constexpr int kReduceFrags = 4;
 __global__ void __launch_bounds__(256) mid_reduce_kernel(const StreamArgs a, int rgw, int mh, int wn) {
-    const int fr = rgw * mh, frags_wg = 2 * wn * fr;
+    const int fr = rgw * mh, frags_wg = 2 * wn * fr;      // fr is a multiple of kReduceFrags (rgw, mh are 2, 4 or 8)
     const int lane = lane_id();
-    const unsigned item = blockIdx.x * 4u + (unsigned)wave_id();      // (tile, wave of the tile, fragment of the wave)
-    const unsigned tile_id = item / (unsigned)frags_wg, rem = item - tile_id * (unsigned)frags_wg;
-    if (tile_id >= (unsigned)(a.n_tiles * a.m_tiles)) return;
-    const int wave = (int)rem / fr, f = (int)rem - wave * fr;
-    const int rg = f / mh, mb = f - rg * mh;
-    const int tile_m = (int)tile_id / a.n_tiles, tile_n = (int)tile_id - tile_m * a.n_tiles;
+    // a workgroup takes 4 * kReduceFrags consecutive fragments of one tile; the workgroups of a weight tile sit on the
+    // XCD that computed it (the grid is n_tiles * m_tiles * chunks workgroups, chunks per tile)
+    const int chunks = (frags_wg + 4 * kReduceFrags - 1) / (4 * kReduceFrags);   // (the last one may have idle waves)
+    int pos;
+    const int tile_n = xcd_weight_tile((int)blockIdx.x, (int)gridDim.x, a.m_tiles * chunks, a.n_tiles, pos);
+    const int tile_m = pos / chunks, chunk = pos - tile_m * chunks;
+    if (tile_n >= a.n_tiles || tile_m >= a.m_tiles) return;
+    const unsigned tile_id = (unsigned)(tile_m * a.n_tiles + tile_n);
+    const unsigned rem = (unsigned)((chunk * 4 + wave_id()) * kReduceFrags);     // (wave of the tile, fragment of the wave)
+    if (rem >= (unsigned)frags_wg) return;
+    const float scale = a.scale ? a.scale[0] : 1.0f;
+    const int wave = (int)rem / fr, f0 = (int)rem - wave * fr;
     const int wq = wave % wn, wm = wave / wn;
     const f32x4* p = reinterpret_cast<const f32x4*>(a.ws + ((size_t)tile_id * a.split_k) * ((size_t)frags_wg * 256) +
-                                                    (size_t)wave * (fr * 256) + (size_t)f * 256) + lane;
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < a.split_k; sp++) v += p[(size_t)sp * ((size_t)frags_wg * 64)];
-    const float scale = a.scale ? a.scale[0] : 1.0f;
+                                                    (size_t)wave * (fr * 256) + (size_t)f0 * 256) + lane;
+    const size_t split_stride = (size_t)frags_wg * 64;
+    f32x4 v[kReduceFrags];
+#pragma unroll
+    for (int j = 0; j < kReduceFrags; j++) v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+    for (int sp = 0; sp < a.split_k; sp++) {
+        f32x4 t[kReduceFrags];
+#pragma unroll
+        for (int j = 0; j < kReduceFrags; j++) t[j] = p[(size_t)sp * split_stride + j * 64];
+#pragma unroll
+        for (int j = 0; j < kReduceFrags; j++) v[j] += t[j];
+    }
     const int r = lane & 15, g = lane >> 4;
-    store_fragment(a, v, scale, tile_m * (32 * mh) + (wm * mh + mb) * 16 + r, tile_n * (16 * rgw * wn) + (wq * rgw + rg) * 16 + 4 * g);
+#pragma unroll
+    for (int j = 0; j < kReduceFrags; j++) {
+        const int f = f0 + j, rg = f / mh, mb = f - rg * mh;
+        store_fragment(a, v[j], scale, tile_m * (32 * mh) + (wm * mh + mb) * 16 + r, tile_n * (16 * rgw * wn) + (wq * rgw + rg) * 16 + 4 * g);
+    }
 }
 
 }  // namespace sg
