@@ -440,11 +440,19 @@ def main():
 
     if args.launch_shapes:
         one = torch.ones(1, device="cuda")
+        if args.calibration_copy:      # what FETCH_SIZE / WRITE_SIZE read for a copy of known size, in the same process
+            src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                dst.copy_(src)
+            torch.cuda.synchronize()
+            del src, dst
         for spec in args.launch_shapes:
             m, n, k = (int(v) for v in spec.lower().split("x"))
             copies = min(6, max(3, int(COLD_BYTES // (n * k)) + 1))
-            wb = [torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8) for _ in range(copies)]
-            a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+            from rocm_dev_amd import synth as _synth
+            wb = [_synth.quantize_tensor(torch.randn((n, k), device="cuda", dtype=torch.float32))[0] for _ in range(copies)]
+            a8 = _synth.quantize_tensor(torch.randn((m, k), device="cuda", dtype=torch.float32))[0]
             d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
             t, _ = sg.skinny_gemm_choice(m, n, k)
             print("%s: %s" % (spec, {f: getattr(t, f) for f in ("engine", "split_k", "waves", "row_tiles", "m_blocks", "depth", "k_chunks",
