@@ -275,7 +275,8 @@ int sg_async_gemm_bf16(const uint8_t* A, const uint8_t* B, void* D_bf16, int m, 
  * B_meta [n][k/8]: one nibble per group - low two bits = position (0..3) of the first kept
  *                  code, high two bits = position of the second (first < second); the group
  *                  with the lower k sits in the low nibble of each byte.
- * k must be a multiple of 512, n even; all pointers 16-byte aligned.  The weights are the
+ * k must be a multiple of 128 and at least 512 (a k that 512 does not divide costs one partly used stage), n even;
+ * all pointers 16-byte aligned.  The weights are the
  * sparse operand of gfx950's v_smfmac_f32_16x16x64_fp8_fp8; HBM traffic is 0.625 bytes per
  * dense weight.  The _tuned form takes row_tiles, waves, depth, split_k and m_blocks from
  * the record (engine 0 = library's choice); wave_tiles = 1 with persistent_wgs_per_cu >= 1

@@ -613,9 +613,14 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
     return c;
 }
 
+// K the 2:4 kernels take: whole 128-k pieces (one lane's share of a 512-k stage; keeps the rows of all three streams
+// 16-byte aligned), at least one whole stage.
+static bool sparse_k_ok(int k) { return k >= 512 && k % 128 == 0; }
+
 // 2:4 sparse engine: c.rg row tiles per wave, c.waves waves splitting K, c.depth ring slots.
 static int launch_sparse_engine(const Config& c, StreamArgs a, const uint8_t* meta, hipStream_t stream) {
-    if (a.k % 512 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (!sparse_k_ok(a.k)) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    const int blocks = (a.k + 511) / 512;   // 512-k stages, the last one partly used when 512 does not divide k
     size_t tiles;
     if (int rc = prepare(c, a, 512, &tiles, stream)) return rc;
     int xu2 = 16;
@@ -630,7 +635,7 @@ static int launch_sparse_engine(const Config& c, StreamArgs a, const uint8_t* me
         // rows, no K split, c.persist workgroups per CU at most
         if (c.mt != 1 || a.m_tiles != 1 || c.split_k != 1 || c.persist < 1 || (c.rg != 1 && c.rg != 2)) return SG_INVALID_CONFIG;
         if (c.waves * 64 > 1024) return SG_TOO_MANY_WARPS;
-        const size_t lds_wt = (size_t)(a.k / 512) * xu2 * 1024 + (size_t)c.waves * c.depth * c.rg * 5120 + 8192;
+        const size_t lds_wt = (size_t)blocks * xu2 * 1024 + (size_t)c.waves * c.depth * c.rg * 5120 + 8192;
         if (lds_wt > 159 * 1024) return SG_INVALID_CONFIG;
         DeviceInfo* dev;
         if (int rc = get_device_info(&dev)) return rc;
@@ -657,7 +662,7 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
     c.split_k = 1;
     c.mt = m <= 16 ? 1 : 2;
     const int tiles16 = (n + 15) / 16;
-    const int blocks = k / 512;
+    const int blocks = (k + 511) / 512;
     // above 8 activation rows the activation stage outweighs a 16-row weight stage: share it between two row tiles
     c.rg = (tiles16 >= 4 * cu_count || (m > 8 && tiles16 >= 2 * cu_count)) ? 2 : 1;
     c.waves = blocks >= 16 ? 2 : 1;
@@ -671,7 +676,7 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
         // 5..16 activation rows and more than one tile per CU: the activation matrix stays resident in LDS and
         // four waves per CU each stream whole tiles (4-33 % faster on ten shapes than refetching 4-8 KB of
         // activations with every 5 KB weight stage; at four rows and below the two are level)
-        const size_t x_res = (size_t)(k / 512) * xu2 * 1024;
+        const size_t x_res = (size_t)blocks * xu2 * 1024;
         for (int depth = 4; depth >= 2; depth--) {
             if (x_res + (size_t)4 * depth * 5120 + 8192 > 159 * 1024) continue;
             c.rg = 1;
@@ -1769,7 +1774,7 @@ int sg_async_gemm_bf16(const uint8_t* A, const uint8_t* B, void* D, int m, int n
 int sg_sparse24_gemm(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D, const float* scale_tensor,
                      int m, int n, int k, void* stream) {
     if (n % 2 != 0) return SG_N_NOT_EVEN;
-    if (k % 512 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (!sparse_k_ok(k)) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (!A || !B_vals || !B_meta || !D || !scale_tensor || m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B_vals) | reinterpret_cast<uintptr_t>(B_meta)) & 15u)
         return SG_BAD_ALIGNMENT;
@@ -1799,7 +1804,7 @@ int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_
                            const float* scale_tensor, int m, int n, int k, const SgTuning* t, void* stream) {
     if (!t) return SG_BAD_ARGUMENT;
     if (n % 2 != 0) return SG_N_NOT_EVEN;
-    if (k % 512 != 0) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
+    if (!sparse_k_ok(k)) return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     if (!A || !B_vals || !B_meta || !D || !scale_tensor || m <= 0 || n <= 0 || k <= 0) return SG_BAD_ARGUMENT;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B_vals) | reinterpret_cast<uintptr_t>(B_meta)) & 15u)
         return SG_BAD_ALIGNMENT;

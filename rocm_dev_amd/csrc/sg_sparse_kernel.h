@@ -20,6 +20,11 @@
 // contiguous bytes per DMA instruction for values and activations, 16 rows x 64 bytes for the
 // metadata - with the 16-byte pieces of each row XOR-swizzled by the row number so that all
 // LDS reads are conflict-free.  HBM traffic per weight row is 0.625 bytes per dense k.
+//
+// K that 512 does not divide (any multiple of 128 from 512 on; builds with TAIL): the last stage is loaded from the
+// window [k - 512, k), which ends with the row, so nothing past a row is read and all three streams stay 16-byte
+// aligned.  The 128-k pieces at the front of that window were already multiplied in the stage before; the lanes that
+// own them (g < 4 - (k % 512) / 128) replace their activation bytes by zeros for that stage.
 #pragma once
 
 #include "sg_device.h"
@@ -38,7 +43,7 @@ struct SparseArgs {
 constexpr int sparse_launch_bound(int MT, int RG) { return (MT == 2 || RG == 4) ? 512 : 1024; }
 
 // XU2 = activation DMA instructions per stage: 2 halves x ceil(rows/4)
-template <int MT, int RG, int XU2, int DEPTH>
+template <int MT, int RG, int XU2, int DEPTH, bool TAIL>
 __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_kernel(const SparseArgs sa) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage]
     __shared__ unsigned arrival;
@@ -60,8 +65,10 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
     const int m0 = tile_m * (16 * MT);
 
     int b_begin, b_end;
-    split_range(a, a.k >> 9, split, b_begin, b_end);   // 512-k stages
+    const int full = a.k >> 9;                          // whole 512-k stages
+    split_range(a, TAIL ? full + 1 : full, split, b_begin, b_end);
     const int mine = blocks_of_wave(a, b_end - b_begin, wave);
+    const int old_pieces = 4 - ((a.k & 511) >> 7);      // TAIL: 128-k pieces of the last window that belong to the stage before
 
     // ---- DMA sources ------------------------------------------------------------------------
     const int v_row = lane >> 4, v_pp = lane & 15;     // values / activations: 4 rows x 16 pieces
@@ -94,16 +101,18 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
     const uint8_t* my_ring = ring + (size_t)wave * (DEPTH * STAGE_BYTES);
     const unsigned my_ring_lds = lds_addr(my_ring);
     auto issue = [&](int i) __attribute__((always_inline)) {
-        const size_t kb = (size_t)(b_begin + wave + i * waves);
+        const int kb = b_begin + wave + i * waves;
+        // first k of the stage: the last stage of a TAIL build starts at k - 512
+        const size_t k0 = (TAIL && kb == full) ? (size_t)a.k - 512 : (size_t)kb << 9;
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) dma_1kb_stream(vsrc[rg][u] + (kb << 8), slot + (rg * 5 + u) * 1024);
-            dma_1kb_stream(tsrc[rg] + (kb << 6), slot + (rg * 5 + 4) * 1024);
+            for (int u = 0; u < 4; u++) dma_1kb_stream(vsrc[rg][u] + (k0 >> 1), slot + (rg * 5 + u) * 1024);
+            dma_1kb_stream(tsrc[rg] + (k0 >> 3), slot + (rg * 5 + 4) * 1024);
         }
 #pragma unroll
-        for (int i2 = 0; i2 < XU2; i2++) dma_1kb(xsrc[i2] + (kb << 9), slot + X_OFF + i2 * 1024);
+        for (int i2 = 0; i2 < XU2; i2++) dma_1kb(xsrc[i2] + k0, slot + X_OFF + i2 * 1024);
     };
 
     // ---- LDS read offsets ---------------------------------------------------------------------
@@ -126,6 +135,14 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
 #pragma unroll
             for (int t = 0; t < 8; t++)
                 x[mt][t] = *reinterpret_cast<const i32x4*>(slot + X_OFF + mt * 8192 + x_rd + (((8 * (g & 1) + t) ^ r) << 4));
+        if constexpr (TAIL) {
+            if (b_begin + wave + i * waves == full && g < old_pieces) {
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                    for (int t = 0; t < 8; t++) x[mt][t] = i32x4{0, 0, 0, 0};
+            }
+        }
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             const uint8_t* w = slot + rg * 5120;
@@ -178,7 +195,7 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
 // tile boundaries.  Tiles are dealt to workgroups first (wave w of workgroup b owns tiles b + G*w,
 // b + G*(w + W), ...), so that with three or four tiles per CU every CU streams; every wave starts its
 // tiles at a K stage of its own and wraps (waves in step at one K offset load the memory channels unevenly).
-template <int RG, int XU2, int DEPTH>
+template <int RG, int XU2, int DEPTH, bool TAIL>
 __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_kernel(const SparseArgs sa) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // X[stages][XU2 KB] | [wave][DEPTH][RG*5 KB] | 8 KB
     const StreamArgs& a = sa.g;
@@ -190,7 +207,10 @@ __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_k
     const int lane = lane_id();
     const int wave = wave_id();
     const int waves = a.waves;
-    const int blocks = a.k >> 9;   // 512-k stages
+    const int full = a.k >> 9;                       // whole 512-k stages
+    const int blocks = TAIL ? full + 1 : full;       // TAIL: one more, loaded from k - 512 and partly used
+    const int old_pieces = 4 - ((a.k & 511) >> 7);
+    auto first_k = [&](int kb) __attribute__((always_inline)) { return (TAIL && kb == full) ? (size_t)a.k - 512 : (size_t)kb << 9; };
     const int first = (int)blockIdx.x + (int)gridDim.x * wave;
     const int stride = (int)gridDim.x * waves;
     const int my_tiles = first < a.n_tiles ? (a.n_tiles - first + stride - 1) / stride : 0;
@@ -213,7 +233,7 @@ __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_k
         for (int i = 0; i < XU2; i++) {
             const int row_l = 4 * (i >> 1) + v_row;
             const int row = row_l < a.m ? row_l : a.m - 1;
-            dma_1kb(a.A + (size_t)row * a.k + ((size_t)kb << 9) + (i & 1) * 256 + ((v_pp ^ (row_l & 15)) << 4),
+            dma_1kb(a.A + (size_t)row * a.k + first_k(kb) + (i & 1) * 256 + ((v_pp ^ (row_l & 15)) << 4),
                     x_lds + (unsigned)(kb * XU2 + i) * 1024);
         }
         x_issued += XU2;
@@ -221,7 +241,7 @@ __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_k
 
     auto issue = [&](int i) __attribute__((always_inline)) {
         const int j = i / blocks;
-        const size_t kb = (size_t)rotated(i - j * blocks);
+        const size_t k0 = first_k(rotated(i - j * blocks));
         const int n0 = (first + j * stride) * (16 * RG);
         const unsigned slot = my_ring_lds + (unsigned)(i % DEPTH) * STAGE_BYTES;
 #pragma unroll
@@ -231,11 +251,11 @@ __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_k
                 const int row16 = 4 * u + v_row;
                 int row = n0 + rg * 16 + row16;
                 row = row < a.n ? row : a.n - 1;   // past the edge: re-read the last row, never stored
-                dma_1kb_stream(a.B + (size_t)row * v_stride + ((v_pp ^ row16) << 4) + (kb << 8), slot + (rg * 5 + u) * 1024);
+                dma_1kb_stream(a.B + (size_t)row * v_stride + ((v_pp ^ row16) << 4) + (k0 >> 1), slot + (rg * 5 + u) * 1024);
             }
             int row = n0 + rg * 16 + t_row;
             row = row < a.n ? row : a.n - 1;
-            dma_1kb_stream(sa.meta + (size_t)row * t_stride + ((t_pp ^ (t_row >> 2)) << 4) + (kb << 6), slot + (rg * 5 + 4) * 1024);
+            dma_1kb_stream(sa.meta + (size_t)row * t_stride + ((t_pp ^ (t_row >> 2)) << 4) + (k0 >> 3), slot + (rg * 5 + 4) * 1024);
         }
     };
 
@@ -251,10 +271,17 @@ __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_k
     int kb_cur = 0;   // stages of the current tile already consumed
     auto consume = [&](int i) __attribute__((always_inline)) {
         const uint8_t* slot = my_ring + (size_t)(i % DEPTH) * STAGE_BYTES;
-        const uint8_t* xs = ring + (size_t)rotated(kb_cur) * (XU2 * 1024);
+        const int kb = rotated(kb_cur);
+        const uint8_t* xs = ring + (size_t)kb * (XU2 * 1024);
         i32x4 x[8];
 #pragma unroll
         for (int t = 0; t < 8; t++) x[t] = *reinterpret_cast<const i32x4*>(xs + x_rd + (((8 * (g & 1) + t) ^ r) << 4));
+        if constexpr (TAIL) {
+            if (kb == full && g < old_pieces) {
+#pragma unroll
+                for (int t = 0; t < 8; t++) x[t] = i32x4{0, 0, 0, 0};
+            }
+        }
 #pragma unroll
         for (int rg = 0; rg < RG; rg++) {
             const uint8_t* w = slot + rg * 5120;

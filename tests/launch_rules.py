@@ -163,15 +163,16 @@ def expect_mid(m, n, k, r):
 
 
 def expect_sparse(m, n, k, r):
-    """2:4 engine: stages of 512 k (5 KB per 16 weight rows: 4 KB of values + 1 KB of metadata)."""
+    """2:4 engine: stages of 512 k (5 KB per 16 weight rows: 4 KB of values + 1 KB of metadata); k in whole 128-k
+    pieces from 512 on, the last stage partly used when 512 does not divide k."""
     waves, rg, mt, depth, sk = r["waves"], r["row_tiles"], r["m_blocks"], r["depth"], r["split_k"]
     persist, wt = r["persistent_wgs_per_cu"], r["wave_tiles"]
-    if k % 512:
+    if k < 512 or k % 128:
         return 3
-    blocks = k // 512
+    full, blocks = k // 512, -(-k // 512)
     if mt not in (1, 2) or wt not in (0, 1):
         return INVALID
-    if not (1 <= waves <= 16 and depth >= 1 and rg >= 1 and 1 <= sk <= blocks):
+    if not (1 <= waves <= 16 and depth >= 1 and rg >= 1 and 1 <= sk <= full):
         return INVALID
     need = (m + 3) // 4
     xu2 = 16 if mt == 2 else (2 if need <= 1 else (4 if need <= 2 else 8))
