@@ -99,8 +99,9 @@ __global__ void __launch_bounds__(1024) ring_gemm_kernel(const RingArgs ra) {
     const int blocks = a.k >> 8;                 // K blocks per tile
     const unsigned ring_lds = lds_addr(ring);
 
-    // The j-th work item of this workgroup: its tile, K split and K range.  Items are numbered with the n tiles
-    // fastest, then the splits of a tile, then the m tiles; the last split takes the remainder of K, so items differ
+    // The j-th work item of this workgroup: its tile, K split and K range.  Items are numbered as decode_tile orders
+    // them - the activation (m) tiles of a weight tile fastest, then the n tiles, then the K splits; the last split
+    // takes the remainder of K, so items differ
     // in length and every role walks them with a cursor over the workgroup's running block count.
     struct Item { int n0, m0, tile_id, split, kb0, cnt; };
     auto item_at = [&](int j) __attribute__((always_inline)) {
