@@ -63,6 +63,10 @@ def main():
     ap.add_argument("--launch-shapes", nargs="+", metavar="MxNxK",
                     help="launch the library's own choice for each dense shape three times, eagerly, on rotating cold weight "
                          "buffers, and exit (for kernel traces and counters of any shape; prints the chosen records)")
+    ap.add_argument("--record", nargs=10, type=int, metavar="INT",
+                    help="with --launch-shapes: launch this tuning record (the ten SgTuning fields: engine split_k waves "
+                         "row_tiles m_blocks depth k_chunks non_temporal persistent_wgs_per_cu wave_tiles) for every shape "
+                         "instead of the library's own choice")
     ap.add_argument("--several-tiles-counters", action="store_true",
                     help="more than 32 rows on small weight matrices (the skinny ring over several 32-row activation tiles): "
                          "launch the library's choice three times each on cold weights and exit (for HBM-traffic counters)")
@@ -96,6 +100,10 @@ def main():
                          "over producers x consumers x b_lanes x qsize) with the library's own choice on the four projection "
                          "shapes at M = 8 and 32, cold weights; then launch each winner and each own choice ten times eagerly "
                          "(for a kernel trace); prints a table, no JSON line")
+    ap.add_argument("--cu-ingest", action="store_true",
+                    help="only run the ingest probe (sg_debug_cu_ingest): what a CU takes in through direct-to-LDS loads from "
+                         "beyond its XCD's L2 (cold), from inside it (hot), and from both at once out of the same or out of "
+                         "different waves, with 16 and with 256 workgroups; prints a table, no JSON line")
     ap.add_argument("--stamps", action="store_true",
                     help="only run the decode GEMMs (four projection shapes at M = --m) back to back from a HIP graph with "
                          "the library's per-workgroup time stamps switched on, and print where a launch period goes "
@@ -116,6 +124,41 @@ def main():
         sys.exit("bench.py: sg_init failed")
     if args.tuning and lib.sg_tuning_load(args.tuning.encode()) != 0:
         sys.exit("bench.py: cannot load tuning table %s" % args.tuning)
+
+    if args.cu_ingest:
+        cold = torch.ones(4 << 30, device="cuda", dtype=torch.uint8)
+        hot = torch.ones(8 << 20, device="cuda", dtype=torch.uint8)       # 1 MB per XCD: stays in its 4 MB L2
+        counts = torch.zeros(2, device="cuda", dtype=torch.int64)
+        ticks = 30000                                                      # 300 us per measurement
+
+        def probe(wgs, waves, cold_waves, hot_per_cold, depth):
+            for timed in (False, True):
+                counts.zero_()
+                rc = lib.sg_debug_cu_ingest(cold.data_ptr(), cold.numel(), hot.data_ptr(), hot.numel(), wgs, waves, cold_waves,
+                                            hot_per_cold, depth, ticks if timed else 3000, counts.data_ptr(), None)
+                if rc != 0:
+                    raise RuntimeError("sg_debug_cu_ingest: %s" % sg.strerror(rc))
+                torch.cuda.synchronize()
+            c, h = (int(v) for v in counts.cpu())
+            per_cu = 1024.0 / wgs / (ticks * 10e-9) / 1e9                  # GB/s per CU and instruction counted
+            return c * per_cu, h * per_cu
+
+        print("direct-to-LDS loads, 1 KB each (8 rows x 128 B), for 300 us; GB/s per CU (x workgroups = chip-wide TB/s)")
+        print("cold = a region of its own per wave (L2 misses), hot = a 1 MB window per XCD shared by its workgroups (L2 hits)")
+        print("| workgroups | waves x loads in flight | stream | cold GB/s | hot GB/s | sum | chip-wide TB/s | cold / cold alone + hot / hot alone |")
+        print("|---|---|---|---|---|---|---|---|")
+        for wgs in (16, 256):
+            for waves, depth in ((4, 8), (8, 8), (16, 8)):
+                alone_c, _ = probe(wgs, waves, waves, 0, depth)
+                _, alone_h = probe(wgs, waves, 0, 0, depth)
+                cases = [("all waves cold", waves, 0), ("all waves hot", 0, 0), ("every wave 1 hot : 1 cold", -1, 1),
+                         ("every wave 3 hot : 1 cold", -1, 3), ("every wave 7 hot : 1 cold", -1, 7),
+                         ("half of the waves cold, half hot", waves // 2, 0), ("a quarter of the waves cold, the others hot", waves // 4, 0)]
+                for name, cw, hpc in cases:
+                    c, h = probe(wgs, waves, cw, hpc, depth)
+                    print("| %d | %d x %d | %s | %.1f | %.1f | %.1f | %.2f | %.2f |"
+                          % (wgs, waves, depth, name, c, h, c + h, (c + h) * wgs / 1e3, c / alone_c + h / alone_h), flush=True)
+        return
 
     if args.n_sweep:
         import ctypes
@@ -454,6 +497,11 @@ def main():
             wb = [_synth.quantize_tensor(torch.randn((n, k), device="cuda", dtype=torch.float32))[0] for _ in range(copies)]
             a8 = _synth.quantize_tensor(torch.randn((m, k), device="cuda", dtype=torch.float32))[0]
             d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+            if args.record:
+                import ctypes
+                forced = sg.SgTuning(*args.record)
+                if lib.sg_tuning_set(m, n, k, ctypes.byref(forced)) != 0:
+                    sys.exit("bench.py: --record is not a valid tuning record")
             t, _ = sg.skinny_gemm_choice(m, n, k)
             print("%s: %s" % (spec, {f: getattr(t, f) for f in ("engine", "split_k", "waves", "row_tiles", "m_blocks", "depth", "k_chunks",
                                                                  "persistent_wgs_per_cu", "wave_tiles")}), file=sys.stderr)

@@ -30,6 +30,17 @@ int sg_debug_stamps(unsigned long long* device_buffer, size_t n_words);
  * 512 (2 rows) or 1024 (1 row). */
 int sg_debug_read_stream(const uint8_t* B, int n, int k, int b_stride, int segment_bytes, void* stream);
 
+/* Profiling aid, no counterpart in the reference: what a CU takes in through direct-to-LDS loads when part of its
+ * stream misses the XCD's L2 and part of it hits.  `workgroups` workgroups of `waves` waves (1, 2, 4, 8 or 16) issue
+ * 1 KB loads (8 rows x 128 B, rows 8 KB apart - the mid-batch GEMM's pattern) with `depth` (4, 8 or 16, at most
+ * 128 / waves) instructions in flight per wave for `ticks` x 10 ns and count them: counts[0] += loads of the cold
+ * stream (a region of its own per wave out of `cold`, streaming hint), counts[1] += loads of the hot stream (one window
+ * per XCD out of `hot`, walked by all its workgroups; make hot_bytes / 8 fit an L2).  cold_waves >= 0: waves below it
+ * stream cold, the others hot; cold_waves < 0: every wave alternates hot_per_cold hot loads with one cold one.
+ * The caller zeroes counts (two 64-bit words in device memory) and reads them after the stream has finished. */
+int sg_debug_cu_ingest(const uint8_t* cold, size_t cold_bytes, const uint8_t* hot, size_t hot_bytes, int workgroups, int waves,
+                       int cold_waves, int hot_per_cold, int depth, int ticks, unsigned long long* counts, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -28,6 +28,7 @@ SIGNATURES = {
     "sg_skinny_gemm_auto_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
     "sg_debug_stamps": (_i, [_vp, _sz]),
     "sg_debug_read_stream": (_i, [_vp, _i, _i, _i, _i, _vp]),
+    "sg_debug_cu_ingest": (_i, [_vp, _sz, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp]),
     "sg_skinny_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "sg_skinny_gemm_fastpath": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "sg_skinny_gemm_auto": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),

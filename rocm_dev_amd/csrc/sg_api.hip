@@ -1370,6 +1370,28 @@ int sg_debug_read_stream(const uint8_t* B, int n, int k, int b_stride, int segme
     return report_hip("read_stream_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
 }
 
+int sg_debug_cu_ingest(const uint8_t* cold, size_t cold_bytes, const uint8_t* hot, size_t hot_bytes, int workgroups, int waves,
+                       int cold_waves, int hot_per_cold, int depth, int ticks, unsigned long long* counts, void* stream) {
+    if (!cold || !hot || !counts || workgroups < 1 || workgroups > 4096 || ticks < 1 || ticks > 1000000) return SG_BAD_ARGUMENT;
+    if (waves != 1 && waves != 2 && waves != 4 && waves != 8 && waves != 16) return SG_BAD_ARGUMENT;
+    if (cold_waves > waves || (cold_waves < 0 && hot_per_cold < 1) || (depth != 4 && depth != 8 && depth != 16)) return SG_BAD_ARGUMENT;
+    if (depth > 128 / waves) return SG_BAD_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(cold) | reinterpret_cast<uintptr_t>(hot)) & 15u) return SG_BAD_ALIGNMENT;
+    // largest powers of two that fit: a region per wave of the cold buffer, one window per XCD of the hot one; a load
+    // instruction spans 8 rows of 8 KB
+    auto floor_pow2 = [](size_t v) { size_t p = 1; while (p * 2 <= v) p *= 2; return p; };
+    const size_t region = floor_pow2(cold_bytes / ((size_t)workgroups * waves)), window = floor_pow2(hot_bytes / 8);
+    if (region < 65536 || window < 65536 || region > 0x80000000u || window > 0x80000000u) return SG_BAD_ARGUMENT;
+    DeviceInfo* dev;
+    if (int rc = get_device_info(&dev)) return rc;
+    auto kernel = depth == 4 ? cu_ingest_kernel<4> : (depth == 8 ? cu_ingest_kernel<8> : cu_ingest_kernel<16>);
+    static LdsGranted granted[3];
+    if (int rc = request_dynamic_lds(reinterpret_cast<const void*>(kernel), 128 * 1024, granted[depth == 4 ? 0 : (depth == 8 ? 1 : 2)])) return rc;
+    kernel<<<dim3((unsigned)workgroups), dim3((unsigned)waves * 64), 128 * 1024, static_cast<hipStream_t>(stream)>>>(
+        cold, (unsigned)region, hot, (unsigned)window, ticks, cold_waves, hot_per_cold, counts);
+    return report_hip("cu_ingest_kernel launch", hipGetLastError()) == hipSuccess ? SG_SUCCESS : SG_LAUNCH_FAILED;
+}
+
 int sg_skinny_gemm(const uint8_t* A, const uint8_t* B, void* D, const float* scale_tensor, int m, int n, int k,
                    int b_stride, int split_k, int A_producers, int B_producers, int consumers, int b_lanes, int qsize,
                    int op_m, int ops, void* stream) {

@@ -52,4 +52,68 @@ __global__ void __launch_bounds__(512) read_stream_kernel(const uint8_t* B, int 
     if (seen == 0x9e3779b9u && sink) *sink = seen;
 }
 
+// Profiling aid: what one CU can take in through direct-to-LDS loads when part of the stream misses the XCD's L2 and
+// part of it hits.  Every wave issues 1 KB loads (8 rows x 128 B, rows 8 KB apart: the mid-batch kernel's pattern)
+// into its own LDS slots, DEPTH instructions in flight, until a wall-clock deadline, and counts them.
+//   cold stream: a region of its own per wave, walked once (streaming hint) - L2 misses
+//   hot stream:  one window per XCD (workgroup id % 8) that all its workgroups walk from different starts - L2 hits
+// cold_waves >= 0: waves [0, cold_waves) stream cold, the others hot.  cold_waves < 0: every wave alternates
+// hot_per_cold hot instructions with one cold one.  counts[0], counts[1]: cold and hot instructions of all workgroups.
+template <int DEPTH>
+__global__ void __launch_bounds__(1024) cu_ingest_kernel(const uint8_t* cold, unsigned cold_region, const uint8_t* hot, unsigned hot_window,
+                                                          int ticks, int cold_waves, int hot_per_cold, unsigned long long* counts) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
+    constexpr unsigned PITCH = 8192;
+    const int lane = lane_id(), wave = wave_id(), waves = (int)blockDim.x >> 6;
+    const int slots = 128 / waves;                                    // 1 KB slots per wave out of 128 KB (waves is a power of two)
+    const unsigned my_lds = lds_addr(ring + (size_t)wave * slots * 1024);
+    const size_t lane_off = (size_t)(lane >> 3) * PITCH + (size_t)(lane & 7) * 16;
+    const uint8_t* cbase = cold + ((size_t)blockIdx.x * waves + wave) * cold_region + lane_off;
+    const uint8_t* hbase = hot + (size_t)(blockIdx.x & 7) * hot_window + lane_off;
+    const unsigned cmask = cold_region - 1, hmask = hot_window - 1;   // both sizes are powers of two, at least 8 rows
+    unsigned cpos = 0, hpos = (unsigned)((((blockIdx.x >> 3) * waves + wave) * 8u * PITCH) & hmask);
+    // along the row in 128-byte steps, then on to the next eight rows, wrapping inside the region
+    auto advance = [](unsigned pos, unsigned mask) __attribute__((always_inline)) {
+        unsigned in_row = (pos & (PITCH - 1)) + 128, grp = pos & ~(PITCH * 8 - 1);
+        if (in_row == PITCH) { in_row = 0; grp += PITCH * 8; }
+        return (grp + in_row) & mask;
+    };
+    int slot = 0;
+    unsigned n_cold = 0, n_hot = 0;
+    auto load_cold = [&]() __attribute__((always_inline)) {
+        dma_1kb_stream(cbase + cpos, my_lds + (unsigned)slot * 1024);
+        cpos = advance(cpos, cmask);
+        slot = (slot + 1) & (slots - 1);
+        n_cold++;
+        wait_vmcnt<DEPTH - 1>();
+    };
+    auto load_hot = [&]() __attribute__((always_inline)) {
+        dma_1kb(hbase + hpos, my_lds + (unsigned)slot * 1024);
+        hpos = advance(hpos, hmask);
+        slot = (slot + 1) & (slots - 1);
+        n_hot++;
+        wait_vmcnt<DEPTH - 1>();
+    };
+    // the clock is read once per batch of loads: a read per load would bound the loop by the read's own latency
+    const unsigned long long t_end = __builtin_amdgcn_s_memrealtime() + (unsigned long long)ticks;
+    if (cold_waves >= 0 && wave < cold_waves) {
+        while (__builtin_amdgcn_s_memrealtime() < t_end)
+            for (int rep = 0; rep < 16; rep++) load_cold();
+    } else if (cold_waves >= 0) {
+        while (__builtin_amdgcn_s_memrealtime() < t_end)
+            for (int rep = 0; rep < 16; rep++) load_hot();
+    } else {
+        while (__builtin_amdgcn_s_memrealtime() < t_end)
+            for (int rep = 0; rep < 4; rep++) {
+                for (int h = 0; h < hot_per_cold; h++) load_hot();
+                load_cold();
+            }
+    }
+    wait_vmcnt<0>();
+    if (lane == 0) {
+        if (n_cold) atomicAdd(&counts[0], n_cold);
+        if (n_hot) atomicAdd(&counts[1], n_hot);
+    }
+}
+
 }  // namespace sg
