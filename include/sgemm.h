@@ -172,10 +172,10 @@ typedef struct SgTuning {
                           3 = the same with the activations in the wavefronts' registers (k = 256 * waves * 1, 2 or 4)
                           (all need persistent_wgs_per_cu >= 1, split_k = 1, m <= 16*m_blocks); + 4 = persistent
                           workgroups get one extra wavefront that streams nothing and does every reduction and store;
-                          8 (alone, with row_tiles = 2, m_blocks = 1, persistent_wgs_per_cu = 0) = 24-row tiles: the
+                          8 (alone, with row_tiles = 2, persistent_wgs_per_cu = 0) = 24-row tiles: the
                           second 16-row fragment carries 8 weight rows (6144 rows = 256 tiles instead of 384);
                           mid-batch: 0 = the last workgroup of a tile to arrive sums the tile's split_k partials, 1 = the
-                          GEMM launch stores partials only and a second launch sums them, one wave per 16 x 16 fragment
+                          GEMM launch stores partials only and a second launch sums them, four 16 x 16 fragments per wave
                           over the whole device (same split order, same result bits); anything else is SG_INVALID_CONFIG */
 } SgTuning;
 

@@ -61,7 +61,7 @@ def lds_ring_fits(m, k, r):
         return False              # part of a block at the end of K: one workgroup per tile, or whole tiles per wave
     blocks = -(-k // 256)
     if r["wave_tiles"] & 8:     # 24-row tiles: two fragments, six weight instructions per stage, one workgroup per tile
-        if r["wave_tiles"] != 8 or r["row_tiles"] != 2 or r["m_blocks"] != 1 or r["persistent_wgs_per_cu"]:
+        if r["wave_tiles"] != 8 or r["row_tiles"] != 2 or r["persistent_wgs_per_cu"]:
             return False
         return ((r["depth"] - 1) * (6 + xu) <= VMCNT_MAX and r["waves"] * r["depth"] * (6 + xu) * 1024 + 4096 <= LDS_USABLE
                 and r["waves"] <= 16 and r["split_k"] <= max(1, blocks))
@@ -152,8 +152,8 @@ def search_space(m, n, k):
             r = record(ENGINE_LDS, sk, waves, rt, mb, depth, 4, 1, persist, wt)
             if lds_ring_fits(m, k, r):
                 out.append(r)
-        for sk, waves, depth in itertools.product((1, 2), (1, 2, 4), (2, 3, 4, 6, 8) if mb == 1 else ()):   # 24-row tiles
-            r = record(ENGINE_LDS, sk, waves, 2, 1, depth, 4, 1, 0, 8)
+        for sk, waves, depth in itertools.product((1, 2), (1, 2, 4), (2, 3, 4, 6, 8) if mb == 1 else (2, 3, 4)):   # 24-row tiles
+            r = record(ENGINE_LDS, sk, waves, 2, mb, depth, 4, 1, 0, 8)
             if lds_ring_fits(m, k, r):
                 out.append(r)
     for ku in (1, 2, 4, 8):

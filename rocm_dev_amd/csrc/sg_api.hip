@@ -319,7 +319,7 @@ static int launch_lds(const Config& c, StreamArgs a, hipStream_t stream) {
         return SG_K_NOT_DIVISIBLE_BY_WARPTILE_K;
     // wave_tiles bit 3: 24-row tiles (two fragments, the second half used), one workgroup per tile
     const bool rows24 = (c.wavetile & 8) != 0;
-    if (rows24 && (c.rg != 2 || c.mt != 1 || c.persist != 0 || (c.wavetile & 7) != 0)) return SG_INVALID_CONFIG;
+    if (rows24 && (c.rg != 2 || c.persist != 0 || (c.wavetile & 7) != 0)) return SG_INVALID_CONFIG;
     size_t tiles;
     if (int rc = prepare(c, a, 256, &tiles, stream, rows24 ? 24 : 0)) return rc;
     // activation DMA instructions per stage: 4 rows each, rounded up to a compiled count

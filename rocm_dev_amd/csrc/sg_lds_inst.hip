@@ -33,7 +33,7 @@ static int launch_one(const StreamArgs& a, unsigned grid, unsigned threads, size
     if (xu == XU_ && depth == DEPTH_) {                                                         \
         if constexpr (XU_ <= 4 * SG_MT && (SG_MT == 1 || XU_ > 4)) {                            \
             if (mode == 5) { /* 24-row tiles: two fragments, six weight instructions per stage */ \
-                if constexpr (SG_MT == 1 && SG_RG == 2 && (DEPTH_ - 1) * (6 + XU_) <= 63)       \
+                if constexpr (SG_RG == 2 && (DEPTH_ - 1) * (6 + XU_) <= 63)                     \
                     return nt ? launch_one<XU_, DEPTH_, true, 5>(a, grid, threads, lds, stream) \
                               : launch_one<XU_, DEPTH_, false, 5>(a, grid, threads, lds, stream); \
                 else                                                                            \

@@ -34,9 +34,9 @@ def expect_lds(m, n, k, r):
     if not (1 <= waves <= 16 and depth >= 1 and rg >= 1 and mt in (1, 2) and 1 <= sk <= blocks):
         return INVALID
     if wt & 8:                                            # 24-row tiles: two fragments, six weight instructions per stage
-        if rg != 2 or mt != 1 or persist != 0 or wt != 8:
+        if rg != 2 or persist != 0 or wt != 8:
             return INVALID
-        per_stage = 6 + activation_instructions(m, 1)
+        per_stage = 6 + activation_instructions(m, mt)
         if waves * depth * per_stage * 1024 + 4096 > LDS_USABLE:
             return INVALID
         if waves * 64 > 1024:

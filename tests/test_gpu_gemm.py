@@ -163,24 +163,23 @@ def test_lds_ring_engine(sg, oracle, cfg, shape):
 
 @pytest.mark.parametrize("cfg", [(1, 1, 8), (1, 2, 4), (2, 1, 4), (1, 4, 2), (3, 2, 3), (1, 1, 6)])
 @pytest.mark.parametrize("shape", [(8, 6144, 4096), (5, 130, 512), (16, 1000, 1024), (8, 50, 256), (1, 24, 768), (13, 6144, 1024),
-                                   (32, 96, 512), (8, 6144, 4224), (13, 100, 640), (9, 200, 1344), (16, 72, 448), (8, 120, 1072), (5, 48, 496)])
+                                   (32, 96, 512), (8, 6144, 4224), (13, 100, 640), (9, 200, 1344), (16, 72, 448), (8, 120, 1072), (5, 48, 496),
+                                   (32, 6144, 4096), (27, 1000, 1024), (17, 50, 768), (32, 130, 1344)])
 def test_lds_ring_24_row_tiles(sg, oracle, cfg, shape):
     """24-row tiles: two 16-row fragments of which the second carries 8 weight rows; its other 8 rows are never fetched
     and never stored (they belong to the next tile).  n a multiple of 24, ragged n (last tile of 10, of 16, of 2 rows),
-    one tile only, K split across workgroups and waves.  m above 16 has no such kernel."""
+    one tile only, K split across workgroups and waves, one and two 16-row activation blocks."""
     split_k, waves, depth = cfg
     m, n, k = shape
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=24)
     ref = gemm_reference(oracle, a8, b8, scale)
     A, B, S = dev(a8), dev(b8), scale_tensor(scale)
     D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
-    kw = dict(engine=2, split_k=split_k, waves=waves, row_tiles=2, m_blocks=1, depth=depth, wave_tiles=8)
+    mb = 1 if m <= 16 else 2
+    kw = dict(engine=2, split_k=split_k, waves=waves, row_tiles=2, m_blocks=mb, depth=depth, wave_tiles=8)
     rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
     torch.cuda.synchronize()
-    want = expect_lds(m, n, k, record(2, split_k, waves, 2, 1, depth, 4, 1, 0, 8)) if m <= 16 else 6
-    if m > 16:
-        kw["m_blocks"] = 2
-        rc = sg.skinny_gemm_tuned(A, B, D, S, **kw)
+    want = expect_lds(m, n, k, record(2, split_k, waves, 2, mb, depth, 4, 1, 0, 8))
     assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
     if rc != 0:
         return   # the refusal asserted above is this case\'s expected result (the configuration does not fit this shape, and the library says so)
