@@ -333,6 +333,8 @@ def main(argv=None):
                     help="keep a shape out of the table unless the winner beats the built-in choice by this fraction "
                          "(negative: always record the winner, even the built-in choice itself)")
     ap.add_argument("--limit", type=int, default=None, help="time only the first N candidates (smoke runs)")
+    ap.add_argument("--report", help="also write what was measured, one JSON object per shape: the built-in choice's and the "
+                                     "winner's microseconds, the winner's record, and whether it went into the table")
     args = ap.parse_args(argv)
     shapes = [tuple(int(x) for x in s.lower().split("x")) for s in args.shapes]
     for p in args.preset:
@@ -340,6 +342,7 @@ def main(argv=None):
     if not shapes:
         ap.error("no shapes: give --shapes and/or --preset")
     entries = parse_table(open(args.merge).read()) if args.merge else {}
+    report = []
     for (m, n, k) in shapes:
         kept, base_us, tried = tune_shape(m, n, k, top=max(1, args.top), launches=args.launches, limit=args.limit)
         print("%dx%dx%d: built-in choice %.2f us; %d candidates ran" % (m, n, k, base_us, tried), flush=True)
@@ -353,8 +356,15 @@ def main(argv=None):
             entries[(m, n, k)] = kept[0][1]
         else:
             entries.pop((m, n, k), None)
+        report.append({"m": m, "n": n, "k": k, "builtin_us": round(base_us, 3), "candidates": tried,
+                       "best_us": round(kept[0][0], 3) if kept else None, "best": kept[0][1] if kept else None,
+                       "best_is_builtin": bool(kept) and same_launch(kept[0][1], own), "in_table": (m, n, k) in entries})
     with open(args.out, "w") as f:
         f.write(format_table(entries.items()))
+    if args.report:
+        import json
+        with open(args.report, "w") as f:
+            f.write("[\n" + ",\n".join(json.dumps(r, sort_keys=True) for r in report) + "\n]\n")
     print("wrote %d record(s) to %s" % (len(entries), args.out))
     return 0
 
