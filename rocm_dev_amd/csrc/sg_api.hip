@@ -496,6 +496,26 @@ static int launch_mid_engine(const Config& c, StreamArgs a, hipStream_t stream) 
     return a.defer_reduce ? launch_mid_reduce(c.rg, c.mt, wn, a, stream) : SG_SUCCESS;
 }
 
+// Microseconds of a mid-batch launch of bn x bm tiles with K split sk ways, from what the ingest probe measured
+// (sg_debug_cu_ingest) rather than from named shapes: a CU takes in operand bytes - L2 misses and hits in turn - at
+// about 55 GB/s with this kernel's mix, the chip serves misses at 6.9 TB/s, the matrix cores sustain about
+// 2 PFLOP/s on real data, and a split adds its partials to every workgroup's stores (27 GB/s per CU), a second launch
+// (4 us) and the partials once more as that launch's reads.
+static double mid_model_us(int m, int n, int k, int bn, int bm, int sk, int cu_count) {
+    const double n_tiles = (n + bn - 1) / bn, m_tiles = (m + bm - 1) / bm;
+    const double wgs = n_tiles * m_tiles * sk;
+    const double rounds = (double)(((long)wgs + cu_count - 1) / cu_count);
+    const double per_wg = (double)(bn + bm) * k / sk / 55e9 + (sk > 1 ? (double)bn * bm * 4 / 27e9 : 0.0);
+    const double hbm = (n_tiles * bn + 8 * m_tiles * bm) * k / 6.9e12;
+    const double mfma = 2.0 * n_tiles * bn * m_tiles * bm * k / 2.0e15;
+    double t = rounds * per_wg;
+    if (hbm > t) t = hbm;
+    if (mfma > t) t = mfma;
+    t += 3.5e-6;
+    if (sk > 1) t += 4.0e-6 + sk * m_tiles * bm * n_tiles * bn * 4 / 6.9e12;
+    return t * 1e6;
+}
+
 // Mid-batch heuristic, fitted to timings of the Llama-3-70B projection shapes at M = 64..256:
 // what matters first is that one round of workgroups covers the device (a second, partly
 // filled round costs more than any tile-shape effect), then that the round is as full as
@@ -571,6 +591,27 @@ static Config pick_mid(int m, int n, int k, int cu_count) {
         }
     }
     Config c = best;
+    // Second opinion of the cost model: a K split over tiles of 128 or 256 weight rows (its sum in a second launch) where
+    // the model puts it at least 8 % ahead of the choice above.  On 72 shapes (64..256 rows x twelve weight shapes) every
+    // override the margin lets through measured level or faster (-27 % ... +0 %: 128 x 5120 x 13824 32.1 -> 23.6 us,
+    // 96 x 9216 x 8192 29.1 -> 23.8, 256 x 8192 x 28672 86.6 -> 77.5), and every choice the model would have made worse
+    // (+4 ... +15 %, all of them ties or within 5 % in the model) stays with the rules.
+    if (k % 128 == 0 && c.waves != 14) {
+        struct Alt { int waves, rg, mt; };
+        static const Alt alts[] = {{4, 2, 2}, {4, 4, 4}, {8, 2, 2}, {8, 2, 4}, {8, 4, 2}, {8, 4, 4}, {8, 2, 8}, {8, 4, 8}};
+        const double own = mid_model_us(m, n, k, 8 * c.rg * c.waves, 32 * c.mt, c.split_k, cu_count);
+        double alt_us = own;
+        for (const Alt& t : alts) {
+            if (32 * t.mt >= 2 * m && t.mt > 2) continue;   // tile more than twice as tall as the problem
+            for (int sk = 2; sk <= 8 && blocks / sk >= 16; sk++) {
+                const double us = mid_model_us(m, n, k, 8 * t.rg * t.waves, 32 * t.mt, sk, cu_count);
+                if (us < alt_us && us <= 0.92 * own) {
+                    alt_us = us;
+                    c.waves = t.waves; c.rg = t.rg; c.mt = t.mt; c.split_k = sk;
+                }
+            }
+        }
+    }
     bool co_resident = false;
     if (m <= 64 && c.waves != 14 && (long)((n + 127) / 128) * 2 >= 3L * cu_count) {
         // memory-bound and many tiles: several small two-slot workgroups per CU hide the DMA
