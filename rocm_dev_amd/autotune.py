@@ -222,11 +222,14 @@ class Bench:
         self.m, self.n, self.k = m, n, k
         g = torch.Generator(device="cuda").manual_seed(seed)
         rot = min(96, max(2, int(640e6 // (n * k)) + 1))
-        # codes 0..119 and 128..247: finite E4M3 of both signs up to 240
+        # N(0, 1) values quantised per tensor to E4M3, the operand distribution of the benchmark configurations: the
+        # large mid-batch launches are power-limited, and uniformly random codes (larger magnitudes on average) rank
+        # their records differently from real data (256 x 57344 x 8192: an eight-wave record 3 % ahead on uniform
+        # codes is 6 % behind on these)
+        from . import synth
+
         def codes(rows):
-            c = torch.randint(0, 120, (rows, k), dtype=torch.uint8, device="cuda", generator=g)
-            s = torch.randint(0, 2, (rows, k), dtype=torch.uint8, device="cuda", generator=g)
-            return c + 128 * s
+            return synth.quantize_tensor(torch.randn((rows, k), device="cuda", dtype=torch.float32, generator=g))[0]
         self.weights = [codes(n) for _ in range(rot)]
         self.A = codes(m)
         self.D = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
