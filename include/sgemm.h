@@ -188,7 +188,9 @@ int sg_skinny_gemm_tuned(const uint8_t* A, const uint8_t* B, void* D_bf16, const
  * device image (8 MB + 4096 counters per GPU, held until the process ends) instead of a workspace from
  * hipMalloc, and nothing is allocated or freed by the call.  A configuration whose partials need more
  * (tiles * split_k * fragment bytes > 8 MB, or more than 4096 output tiles with split_k > 1) is refused
- * with SG_WORKSPACE_TOO_SMALL; without a K split there is no limit.  The counters are cleared by a kernel with
+ * with SG_WORKSPACE_TOO_SMALL; without a K split there is no limit.  With engine = 0 the library's own choice is made
+ * to fit: a K split that does not fit the array is not taken (the result then differs from sg_skinny_gemm_tuned's in
+ * summation order only).  The counters are cleared by a kernel with
  * the first call on a device; after that every launch that completes leaves them zero.  All calls on one GPU share the array:
  * calls that overlap on one GPU (two streams, unordered graph nodes) race, calls in stream order do not. */
 int sg_skinny_gemm_tuned_noalloc(const uint8_t* A, const uint8_t* B, void* D_bf16, const float* scale_tensor,

@@ -1528,7 +1528,16 @@ int sg_skinny_gemm_tuned_noalloc(const uint8_t* A, const uint8_t* B, void* D, co
     bool first_use = false;
     if (int rc = static_workspace(&w, &first_use)) return rc;
     Config c = config_from_tuning(*t);
-    if (c.engine == ENGINE_AUTO) c = heuristic_config(m, n, k, dev->cu_count);
+    if (c.engine == ENGINE_AUTO) {
+        c = heuristic_config(m, n, k, dev->cu_count);
+        // the library's own choice is made to fit the array: a K split whose partials or counters do not, is not taken
+        size_t partial_bytes, counters;
+        workspace_need(c, m, n, &partial_bytes, &counters);
+        if (partial_bytes > w.partial_bytes || counters > w.n_counters) {
+            c.split_k = 1;
+            if (c.engine == ENGINE_MID) c.wavetile = 0;
+        }
+    }
     if (c.engine != ENGINE_MID && c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
     c.fixed_ws = &w;
     StreamArgs a{};

@@ -59,6 +59,28 @@ def test_noalloc_matches_tuned_on_two_calls_in_a_row(sg, oracle, pair):
             assert oracle.max_rel_err_bf16(bits(got), ref) <= GEMM_TOL
 
 
+def test_noalloc_own_choice_is_made_to_fit_the_array(sg, oracle):
+    """engine = 0 on a shape for which the library would split K with more partials than the array holds (128 x 10240 x
+    8192: three splits of 128 x 128 tiles, 15.7 MB): the split is not taken, the call succeeds and allocates nothing."""
+    m, n, k = 128, 10240, 8192
+    choice, _ = sg.skinny_gemm_choice(m, n, k)
+    assert choice.engine == 4 and choice.split_k > 1
+    a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=5)
+    A, B, S = dev(a8), dev(b8), scale_tensor(scale)
+    want = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_tuned(A, B, want, S, engine=0) == 0
+    gc.collect()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated(), sg.workspace_bytes()
+    rc = sg.skinny_gemm_tuned_noalloc(A, B, got, S, engine=0)
+    assert rc == 0, sg.strerror(rc)
+    torch.cuda.synchronize()
+    assert (torch.cuda.memory_allocated(), sg.workspace_bytes()) == before
+    # another summation order than the split launch: equal to the GEMM tolerance, not bit for bit
+    assert oracle.max_rel_err_bf16(bits(got), bits(want)) <= GEMM_TOL
+
+
 def test_noalloc_refuses_partials_beyond_its_array(sg, oracle):
     """8 MB of partials, 4096 counters: a 4-way split of 256 x 8192 tiles of 128 x 128 needs 64 * 2 * 4 * 64 KB."""
     m, n, k = 256, 8192, 8192
