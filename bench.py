@@ -80,8 +80,9 @@ def main():
     ap.add_argument("--sparse-counters", action="store_true",
                     help="only launch the 2:4 GEMMs (14336 x 4096 and 28672 x 4096 at M = 8, 16; then 4096 x 14336 at M = 8, 16, 32 through the library's choice only), eagerly, three times each "
                          "on cold weights through the library's choice and three times through the one-wave-workgroup kernel "
-                         "it replaced, after three 256 MiB copies of known traffic, and exit (for L2 / HBM traffic counter runs; "
-                         "prints no JSON line)")
+                         "it replaced, after three 256 MiB copies of known traffic (for L2 / HBM traffic counter runs); then "
+                         "graph-times K = 4224, 4480, 14464, 14720 - whole 128-k pieces that 512 does not divide - next to "
+                         "the neighbouring multiples of 512 and prints that table; no JSON line")
     ap.add_argument("--k-tail-counters", action="store_true",
                     help="K that 256 does not divide: launch the library's choice (LDS ring with a partly used last stage) and the "
                          "register-streaming engine it replaced three times each on cold weights, next to the neighbouring "
@@ -479,6 +480,50 @@ def main():
                 if rc != 0:
                     raise RuntimeError("sg_sparse24_gemm: %s" % sg.strerror(rc))
             torch.cuda.synchronize()
+        # K that 512 does not divide next to its neighbours: graph-timed on cold weights (prints a table)
+        side = torch.cuda.Stream()
+        print("2:4 GEMM, K in whole 128-k pieces that 512 does not divide, us per launch (cold weights, graphs of 32 launches)")
+        print("| M | N | " + " | ".join("K = %d" % kk for kk in (4096, 4224, 4480, 4608)) + " | N | " +
+              " | ".join("K = %d" % kk for kk in (14336, 14464, 14720, 14848)) + " |")
+        print("|---|---|---|---|---|---|---|---|---|---|---|")
+        for m in (8, 16, 32):
+            cells = []
+            for n, ks in ((14336, (4096, 4224, 4480, 4608)), (4096, (14336, 14464, 14720, 14848))):
+                cells.append(str(n))
+                for kk in ks:
+                    vb, mb = [], []
+                    for _ in range(8):
+                        dense = torch.randint(0, 0x7E, (n, kk), device="cuda", dtype=torch.uint8)
+                        v = torch.empty((n, kk // 2), device="cuda", dtype=torch.uint8)
+                        t = torch.empty((n, kk // 8), device="cuda", dtype=torch.uint8)
+                        if lib.sg_sparse24_compress(dense.data_ptr(), v.data_ptr(), t.data_ptr(), n, kk, kk, None) != 0:
+                            raise RuntimeError("sg_sparse24_compress failed")
+                        vb.append(v)
+                        mb.append(t)
+                    del dense
+                    a8 = torch.randint(0, 0x7E, (m, kk), device="cuda", dtype=torch.uint8)
+                    d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+                    with torch.cuda.stream(side):
+                        g = torch.cuda.CUDAGraph()
+                        with torch.cuda.graph(g, stream=side):
+                            st = torch.cuda.current_stream().cuda_stream
+                            for i in range(32):
+                                rc = lib.sg_sparse24_gemm(a8.data_ptr(), vb[i % 8].data_ptr(), mb[i % 8].data_ptr(), d.data_ptr(),
+                                                          one.data_ptr(), m, n, kk, st)
+                                if rc != 0:
+                                    raise RuntimeError("sg_sparse24_gemm: %s" % sg.strerror(rc))
+                        ts = []
+                        for r in range(12):
+                            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                            e0.record()
+                            g.replay()
+                            e1.record()
+                            torch.cuda.synchronize()
+                            if r >= 3:
+                                ts.append(e0.elapsed_time(e1) * 1e3 / 32)
+                    cells.append("%.2f" % sorted(ts)[len(ts) // 2])
+                    del vb, mb, g
+            print("| %d | " % m + " | ".join(cells) + " |", flush=True)
         return
 
     if args.launch_shapes:
