@@ -368,10 +368,12 @@ def test_producer_consumer_ring_split_k(sg, oracle, cfg, shape, split_k):
 
 
 @pytest.mark.parametrize("shape", [(8, 4096, 4096), (5, 130, 512), (32, 6144, 1024), (16, 28672, 1024), (64, 512, 1024),
-                                   (200, 258, 2048), (1, 64, 48), (256, 1024, 512)])
+                                   (200, 258, 2048), (1, 64, 48), (256, 1024, 512),
+                                   (96, 5120, 13824), (100, 3002, 8192)])   # the last two: K split, sum (and factors) in the second launch
 @pytest.mark.parametrize("which", ["both", "rows", "cols", "none"])
 def test_row_and_column_scaled_epilogue(sg, oracle, shape, which):
-    """sg_skinny_gemm_rowcol: scalar, per-activation-row and per-output-column factors in the epilogue."""
+    """sg_skinny_gemm_rowcol: scalar, per-activation-row and per-output-column factors in the epilogue - of the GEMM
+    kernels and of the launch that sums a mid-batch K split."""
     m, n, k = shape
     a8, b8, scale = oracle.make_gemm_operands(m, n, k, seed=31)
     rng = np.random.default_rng(m + n + k)
