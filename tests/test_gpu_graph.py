@@ -32,6 +32,9 @@ def test_replays_match_eager(oracle):
     jobs.append(("split-K ring", *gemm(32, 512, 14336, 4, dict(engine=2, split_k=2, waves=2, row_tiles=2, depth=3))))
     jobs.append(("mid", *gemm(128, 1024, 2048, 5)))
     jobs.append(("mid split-K", *gemm(64, 512, 8192, 6, dict(engine=4, split_k=2, waves=8, row_tiles=2, m_blocks=2, depth=4, k_chunks=2))))
+    jobs.append(("mid split-K, sum in a second launch", *gemm(64, 512, 8192, 14, dict(engine=4, split_k=2, waves=8, row_tiles=2, m_blocks=2,
+                                                                               depth=4, k_chunks=2, wave_tiles=1))))
+    jobs.append(("mid, the library's own six-way split and second launch", *gemm(96, 5120, 13824, 15)))
     # the library's own choices with a K split, several activation tiles, whole tiles per wave and a partial last K block
     jobs.append(("several activation tiles, two K splits", *gemm(40, 1024, 16384, 9)))
     jobs.append(("whole tiles per wave", *gemm(8, 20480, 512, 10)))
