@@ -2,10 +2,13 @@
 output against torch's dequantise-to-fp32 matmul (rocBLAS, a different summation order, no code shared with
 the library or the oracle), and against torch._scaled_mm (hipBLASLt's own FP8 path) where this torch build
 has it.  The oracle-based tests cover slices of these shapes; this covers every tile of them."""
+import random
+
 import pytest
 import torch
 
 from gpu_util import GEMM_TOL
+from rocm_dev_amd.api import ENGINE_MID
 
 pytestmark = pytest.mark.gpu
 
@@ -37,13 +40,14 @@ def _metric(d, ref):
     return float(((d - ref).abs() / ref.abs().clamp_min(floor)).max())
 
 
-def _dequant_matmul(A, B, S, chunk=8192):
-    """fp32 matmul of the decoded operands, weight rows in chunks to bound the fp32 copy."""
+def _dequant_matmul(A, B, S, chunk=8192, rounded=True):
+    """fp32 matmul of the decoded operands, weight rows in chunks to bound the fp32 copy; rounded to bf16 like the
+    library's output, or left in fp32."""
     a = A.float()
     out = torch.empty((A.shape[0], B.shape[0]), dtype=torch.float32, device="cuda")
     for lo in range(0, B.shape[0], chunk):
         out[:, lo:lo + chunk] = a @ B[lo:lo + chunk].float().t()
-    return (out * S).bfloat16()
+    return (out * S).bfloat16() if rounded else out * S
 
 
 @pytest.mark.parametrize("n,k", DECODE)
@@ -64,6 +68,59 @@ def test_mid_batch_shapes_against_torch_fp32(sg, m, n, k):
     assert sg.skinny_gemm_fastpath(A, B, D, S) == 0
     torch.cuda.synchronize()
     assert _metric(D, _dequant_matmul(A, B, S)) <= GEMM_TOL
+
+
+def _split_decision_cases(count=32):
+    """Seeded shapes in the range where the library weighs a K split, summed by a second launch, against an unsplit
+    launch: 33..256 rows, K a multiple of 128 (every fourth: of 64 only, so the last K block is partly used); three in
+    four with 2048..16384 weight rows, the others with 1024..4096, where too few tiles fill the device."""
+    rng = random.Random(50331)
+    cases = []
+    for i in range(count):
+        n = 2 * (rng.randint(512, 2048) if i % 4 == 1 else rng.randint(1024, 8192))
+        cases.append((rng.randint(33, 256), n, 128 * rng.randint(16, 128) + (64 if i % 4 == 3 else 0)))
+    return cases
+
+
+def _kind_of_launch(sg, m, n, k):
+    t, _ = sg.skinny_gemm_choice(m, n, k)
+    if t.split_k == 1:
+        return "unsplit"
+    return "second launch sums" if t.engine == ENGINE_MID and t.wave_tiles == 1 else "last workgroup sums"
+
+
+@pytest.mark.parametrize("m,n,k", _split_decision_cases())
+def test_split_decision_shapes_against_torch_fp32(sg, m, n, k):
+    """Whatever the library decides for the shape, the whole output matches the fp32 matmul, and the same decision
+    run on a caller-owned workspace returns the same bits.
+
+    The matmul is left in fp32 here, so the bar holds one bf16 rounding, the library's.  The metric's floor, 1e-2 of
+    the output's rms, is 130 bf16 steps of a value just under it, so the bar is a step and a quarter there: on
+    143 x 2374 x 5440 one output of 0.5529 (floor 0.736) comes out as 0.546875 where the rounded matmul says 0.5546875,
+    two steps apart or 0.0106 - with bits equal to the oracle's model of the matrix instruction's summation on every
+    engine of the library - and 0.0082 from the unrounded value."""
+    A, B, S = _operands(m, n, k, seed=m + n + k)
+    D = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_fastpath(A, B, D, S) == 0
+    torch.cuda.synchronize()
+    assert _metric(D, _dequant_matmul(A, B, S, rounded=False)) <= GEMM_TOL, _kind_of_launch(sg, m, n, k)
+    need = sg.workspace_query(m, n, k)
+    assert (need > 0) == (_kind_of_launch(sg, m, n, k) != "unsplit")
+    ws = None
+    if need:
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        sg.workspace_init(ws)
+    D2 = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert sg.skinny_gemm_auto_ws(A, B, D2, S, ws) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(D.view(torch.int16), D2.view(torch.int16))
+
+
+def test_split_decision_shapes_reach_split_and_unsplit_launches(sg):
+    """The seeded shapes above are worth their time only if both decisions occur among them, with and without a partly
+    used last K block (from 33 rows on a split chosen by the library is always summed by a second launch)."""
+    seen = {(_kind_of_launch(sg, m, n, k), k % 128 == 0) for m, n, k in _split_decision_cases()}
+    assert seen == {(kind, whole) for kind in ("unsplit", "second launch sums") for whole in (True, False)}
 
 
 @pytest.mark.parametrize("n,k", [(4096, 14336), (14336, 4096)])
