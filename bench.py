@@ -83,6 +83,11 @@ def main():
                          "it replaced, after three 256 MiB copies of known traffic (for L2 / HBM traffic counter runs); then "
                          "graph-times K = 4224, 4480, 14464, 14720 - whole 128-k pieces that 512 does not divide - next to "
                          "the neighbouring multiples of 512 and prints that table; no JSON line")
+    ap.add_argument("--sparse-metadata-fetch", action="store_true",
+                    help="only compare the two ways the 2:4 kernels fetch their metadata on the 4096 x 14336 and 14336 x 4096 "
+                         "shapes at M = 1, 8, 16, 32: by 64-byte pieces per row and stage, and by whole 128-byte lines per "
+                         "row and pair of stages; three eager launches of each on cold weights (for L1 -> L2 request "
+                         "counters), then alternating graph replays; prints a table, no JSON line")
     ap.add_argument("--k-tail-counters", action="store_true",
                     help="K that 256 does not divide: launch the library's choice (LDS ring with a partly used last stage) and the "
                          "register-streaming engine it replaced three times each on cold weights, next to the neighbouring "
@@ -420,6 +425,79 @@ def main():
                         raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
                 torch.cuda.synchronize()
             del wb
+        return
+
+    if args.sparse_metadata_fetch:
+        import ctypes
+        one = torch.ones(1, device="cuda")
+        side = torch.cuda.Stream()
+        copies = 8
+        # the records the library chooses for these shapes (engine, split_k, waves, row_tiles, m_blocks, depth, k_chunks,
+        # non_temporal, persistent_wgs_per_cu, wave_tiles), written out so that k_chunks can say how the metadata is
+        # fetched: 1 = by pieces, 8 = by lines.  (16 x 14336 x 4096: three slots - four do not fit next to the lines' ring.)
+        cases = [(1, 14336, 4096, (2, 1, 1, 1, 1, 2, 0, 1, 0, 0)), (8, 14336, 4096, (2, 1, 4, 1, 1, 4, 0, 1, 1, 1)),
+                 (16, 14336, 4096, (2, 1, 4, 1, 1, 3, 0, 1, 1, 1)), (32, 14336, 4096, (2, 1, 1, 2, 2, 2, 0, 1, 0, 0)),
+                 (1, 4096, 14336, (2, 1, 2, 1, 1, 4, 0, 1, 0, 0)), (8, 4096, 14336, (2, 1, 2, 1, 1, 4, 0, 1, 0, 0)),
+                 (16, 4096, 14336, (2, 1, 2, 1, 1, 4, 0, 1, 0, 0)), (32, 4096, 14336, (2, 1, 2, 1, 2, 3, 0, 1, 0, 0))]
+        print("2:4 GEMM, metadata by 64-byte pieces per stage against whole 128-byte lines per pair of stages, us per launch "
+              "(cold weights, graphs of %d launches, alternating replays, medians of 12)" % (4 * copies))
+        print("| M x N x K | waves, row tiles, slots | pieces | lines | lines / pieces |")
+        print("|---|---|---|---|---|")
+        weights = {}
+        for m, n, k, fields in cases:
+            if (n, k) not in weights:
+                weights.clear()
+                vb, mb = [], []
+                for _ in range(copies):
+                    dense = torch.randint(0, 0x7E, (n, k), device="cuda", dtype=torch.uint8)
+                    v = torch.empty((n, k // 2), device="cuda", dtype=torch.uint8)
+                    t = torch.empty((n, k // 8), device="cuda", dtype=torch.uint8)
+                    if lib.sg_sparse24_compress(dense.data_ptr(), v.data_ptr(), t.data_ptr(), n, k, k, None) != 0:
+                        raise RuntimeError("sg_sparse24_compress failed")
+                    vb.append(v)
+                    mb.append(t)
+                    del dense
+                weights[(n, k)] = (vb, mb)
+            vb, mb = weights[(n, k)]
+            a8 = torch.randint(0, 0x7E, (m, k), device="cuda", dtype=torch.uint8)
+            d = torch.empty((m, n), device="cuda", dtype=torch.bfloat16)
+            recs = {}
+            for kc in (1, 8):
+                f = list(fields)
+                f[6] = kc
+                recs[kc] = sg.SgTuning(*f)
+
+            def launch(kc, i, stream):
+                rc = lib.sg_sparse24_gemm_tuned(a8.data_ptr(), vb[i % copies].data_ptr(), mb[i % copies].data_ptr(), d.data_ptr(),
+                                                one.data_ptr(), m, n, k, ctypes.byref(recs[kc]), stream)
+                if rc != 0:
+                    raise RuntimeError("sg_sparse24_gemm_tuned: %s" % sg.strerror(rc))
+
+            for kc in (1, 8):           # for the counters: three cold launches of each
+                for i in range(3):
+                    launch(kc, 3 * (kc // 8) + i, None)
+                torch.cuda.synchronize()
+            graphs = {}
+            with torch.cuda.stream(side):
+                for kc in (1, 8):
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g, stream=side):
+                        for i in range(4 * copies):
+                            launch(kc, i, torch.cuda.current_stream().cuda_stream)
+                    graphs[kc] = g
+                times = {1: [], 8: []}
+                for rep in range(14):
+                    for kc in (1, 8):
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record()
+                        graphs[kc].replay()
+                        e1.record()
+                        torch.cuda.synchronize()
+                        if rep >= 2:
+                            times[kc].append(e0.elapsed_time(e1) * 1e3 / (4 * copies))
+            med = {kc: sorted(v)[len(v) // 2] for kc, v in times.items()}
+            print("| %d x %d x %d | %d, %d, %d%s | %.2f | %.2f | %.3f |" % (m, n, k, fields[2], fields[3], fields[5],
+                  ", wave per tile" if fields[9] else "", med[1], med[8], med[8] / med[1]), flush=True)
         return
 
     if args.sparse_counters:

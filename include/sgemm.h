@@ -283,7 +283,10 @@ int sg_async_gemm_bf16(const uint8_t* A, const uint8_t* B, void* D_bf16, int m, 
  * dense weight.  The _tuned form takes row_tiles, waves, depth, split_k and m_blocks from
  * the record (engine 0 = library's choice); wave_tiles = 1 with persistent_wgs_per_cu >= 1
  * selects the kernel that keeps the activation matrix resident in LDS and gives every wave
- * whole 16*row_tiles-row tiles (m <= 16, split_k = 1, row_tiles 1 or 2). */
+ * whole 16*row_tiles-row tiles (m <= 16, split_k = 1, row_tiles 1 or 2).  Where k is a multiple of 1024 (and
+ * split_k <= k / 1024) the metadata is fetched by whole 128-byte lines, two K stages per row and request, as long as
+ * the ring that takes (4 KB of LDS per wave and row tile more) fits; k_chunks = 1 in the record keeps the fetch by
+ * 64-byte pieces per stage. */
 int sg_sparse24_gemm(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D_bf16,
                      const float* scale_tensor, int m, int n, int k, void* stream);
 int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_t* B_meta, void* D_bf16,

@@ -671,26 +671,37 @@ static int launch_sparse_engine(const Config& c, StreamArgs a, const uint8_t* me
     }
     SparseArgs sa;
     sa.meta = meta;
+    // Metadata by whole 128-byte lines (two stages' worth per row and request) where K is a multiple of 1024, every K
+    // split holds whole pairs of stages and the pair ring still fits the LDS; by 64-byte pieces per stage otherwise, or
+    // when the record asks for that (k_chunks = 1).
+    const size_t pair_ring = (size_t)(c.depth / 2 + 2) * c.rg * 2048;   // per wave, in place of depth x rg KB
+    bool pairs = c.ku != 1 && a.k % 1024 == 0 && c.split_k <= a.k / 1024;
     if (c.wavetile == 1) {
         // every wave owns whole tiles, the activation matrix is resident in LDS: one activation tile of at most 16
         // rows, no K split, c.persist workgroups per CU at most
         if (c.mt != 1 || a.m_tiles != 1 || c.split_k != 1 || c.persist < 1 || (c.rg != 1 && c.rg != 2)) return SG_INVALID_CONFIG;
         if (c.waves * 64 > 1024) return SG_TOO_MANY_WARPS;
-        const size_t lds_wt = (size_t)blocks * xu2 * 1024 + (size_t)c.waves * c.depth * c.rg * 5120 + 8192;
+        size_t lds_wt = (size_t)blocks * xu2 * 1024 + (size_t)c.waves * c.depth * c.rg * 5120 + 8192;
         if (lds_wt > 159 * 1024) return SG_INVALID_CONFIG;
+        const size_t lds_pairs = (size_t)blocks * xu2 * 1024 + (size_t)c.waves * (c.depth * c.rg * 4096 + pair_ring) + 8192;
+        pairs = pairs && lds_pairs <= 159 * 1024;
+        if (pairs) lds_wt = lds_pairs;
         DeviceInfo* dev;
         if (int rc = get_device_info(&dev)) return rc;
         size_t grid = (size_t)dev->cu_count * c.persist;
         if (grid > tiles) grid = tiles;
         sa.g = a;
-        return launch_sparse_wavetile(c.rg, xu2, c.depth, sa, (unsigned)grid, (unsigned)c.waves * 64, lds_wt, stream);
+        return launch_sparse_wavetile(c.rg, xu2, c.depth, pairs, sa, (unsigned)grid, (unsigned)c.waves * 64, lds_wt, stream);
     }
     const size_t stage = (size_t)(c.rg * 5 + xu2) * 1024;
     // + 8 KB: lanes of activation rows that are not loaded read past the last slot
-    const size_t lds = (size_t)c.waves * c.depth * stage + 8192;
+    size_t lds = (size_t)c.waves * c.depth * stage + 8192;
     if (lds > 159 * 1024) return SG_INVALID_CONFIG;
+    const size_t lds_pairs = (size_t)c.waves * (c.depth * (stage - (size_t)c.rg * 1024) + pair_ring) + 8192;
+    pairs = pairs && lds_pairs <= 159 * 1024;
+    if (pairs) lds = lds_pairs;
     sa.g = a;
-    return launch_sparse(c.mt, c.rg, xu2, c.depth, sa, (unsigned)(tiles * c.split_k), (unsigned)c.waves * 64, lds, stream);
+    return launch_sparse(c.mt, c.rg, xu2, c.depth, pairs, sa, (unsigned)(tiles * c.split_k), (unsigned)c.waves * 64, lds, stream);
 }
 
 static Config pick_sparse(int m, int n, int k, int cu_count) {
@@ -717,9 +728,12 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
         // 5..16 activation rows and more than one tile per CU: the activation matrix stays resident in LDS and
         // four waves per CU each stream whole tiles (4-33 % faster on ten shapes than refetching 4-8 KB of
         // activations with every 5 KB weight stage; at four rows and below the two are level)
+        // (a K of whole 1024s gets its metadata by lines, which takes a pair ring next to the stages: at 9..16 rows and
+        // K = 4096 three stages with it, 9.0-9.1 us on 16 x 14336 x 4096, rather than four without, 9.3)
         const size_t x_res = (size_t)blocks * xu2 * 1024;
         for (int depth = 4; depth >= 2; depth--) {
-            if (x_res + (size_t)4 * depth * 5120 + 8192 > 159 * 1024) continue;
+            const size_t wave_bytes = k % 1024 == 0 ? (size_t)depth * 4096 + (size_t)(depth / 2 + 2) * 2048 : (size_t)depth * 5120;
+            if (x_res + 4 * wave_bytes + 8192 > 159 * 1024) continue;
             c.rg = 1;
             c.waves = 4;
             c.depth = depth;
@@ -728,6 +742,10 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
             break;
         }
     }
+    // Metadata by whole lines (launch_sparse_engine) costs a wave 4 KB of LDS more: with one-wave workgroups on
+    // two-slot rings that is one workgroup less per CU, and up to 4 activation rows it does not pay (1 x 14336 x 4096
+    // 7.9 -> 8.0 us, where 32 x 14336 x 4096 on the same ring goes 12.7 -> 12.0 and 16 x 4096 x 14336 11.7 -> 10.2)
+    if (m <= 4 && c.depth == 2 && c.waves == 1) c.ku = 1;
     return c;
 }
 
@@ -1892,6 +1910,7 @@ int sg_sparse24_gemm_tuned(const uint8_t* A, const uint8_t* B_vals, const uint8_
         c.mt = t->m_blocks;
         c.persist = t->persistent_wgs_per_cu;
         c.wavetile = t->wave_tiles;
+        c.ku = t->k_chunks;   // 1: metadata by 64-byte pieces per stage also where whole lines are possible
         if (c.mt != 1 && c.mt != 2) return SG_INVALID_CONFIG;
         if (c.wavetile != 0 && c.wavetile != 1) return SG_INVALID_CONFIG;
     }

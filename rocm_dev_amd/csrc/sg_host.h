@@ -49,10 +49,10 @@ int launch_mid(int rgw, int mh, int depth, int dx, int wn, const StreamArgs& a, 
 int launch_mid_reduce(int rgw, int mh, int wn, const StreamArgs& a, hipStream_t stream);
 
 struct SparseArgs;
-int launch_sparse(int mt, int rg, int xu2, int depth, const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds,
-                  hipStream_t stream);
-int launch_sparse_wavetile(int rg, int xu2, int depth, const SparseArgs& sa, unsigned grid, unsigned threads, size_t lds,
-                           hipStream_t stream);
+int launch_sparse(int mt, int rg, int xu2, int depth, bool pairs, const SparseArgs& sa, unsigned grid, unsigned threads,
+                  size_t lds, hipStream_t stream);
+int launch_sparse_wavetile(int rg, int xu2, int depth, bool pairs, const SparseArgs& sa, unsigned grid, unsigned threads,
+                           size_t lds, hipStream_t stream);
 
 // Prints a HIP failure to stderr when the environment variable SG_VERBOSE is set; returns e.
 hipError_t report_hip(const char* what, hipError_t e);

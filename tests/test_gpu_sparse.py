@@ -91,15 +91,24 @@ SPARSE_CONFIGS = [
 ]
 
 
+# k_chunks of a 2:4 record: 1 = metadata fetched per stage in 64-byte pieces also where K (a multiple of 1024) allows
+# whole 128-byte lines per pair of stages; anything else = by lines where possible
+METADATA_FETCH = [8, 1]
+
+
+@pytest.mark.parametrize("k_chunks", METADATA_FETCH)
 @pytest.mark.parametrize("cfg", SPARSE_CONFIGS)
-@pytest.mark.parametrize("shape", [(8, 512, 4096), (16, 200, 2048), (32, 256, 2048), (5, 4096, 1024),
+@pytest.mark.parametrize("shape", [(8, 512, 4096), (16, 200, 2048), (32, 256, 2048), (5, 4096, 1024), (3, 6, 3072), (27, 42, 3072),
                                    (8, 512, 4224), (32, 200, 1920), (13, 1000, 640)])   # the last three: K that 512 does not divide
-def test_sparse_tuned_configs(sg, oracle, cfg, shape):
+def test_sparse_tuned_configs(sg, oracle, cfg, shape, k_chunks):
+    """K splits and waves sharing K by stages or, with the metadata fetched by lines, by pairs of stages: one pair per
+    split (4096 split four ways over two row tiles), an odd number of pairs over two waves (3072), fewer weight rows
+    than half a tile (n = 6: the lines of rows 8..15 are the last row's again)."""
     split_k, waves, row_tiles, depth = cfg
     m, n, k = shape
     a8, vals, meta, b8, scale = oracle.make_sparse24_operands(m, n, k, seed=21)
     ref = sparse_reference(oracle, a8, vals, meta, scale)
-    t = sg.SgTuning(2, split_k, waves, row_tiles, 1 if m <= 16 else 2, depth, 8, 1, 0)
+    t = sg.SgTuning(2, split_k, waves, row_tiles, 1 if m <= 16 else 2, depth, k_chunks, 1, 0)
     rc, got = _run(sg, a8, vals, meta, scale, tuning=t)
     want = expect_sparse(m, n, k, record(2, split_k, waves, row_tiles, 1 if m <= 16 else 2, depth))
     assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
@@ -121,17 +130,19 @@ WAVETILE_CONFIGS = [
 ]
 
 
+@pytest.mark.parametrize("k_chunks", METADATA_FETCH)
 @pytest.mark.parametrize("cfg", WAVETILE_CONFIGS)
-@pytest.mark.parametrize("shape", [(8, 14336, 4096), (1, 4096, 1024), (5, 1000, 1024), (16, 6000, 2048), (13, 200, 512),
+@pytest.mark.parametrize("shape", [(8, 14336, 4096), (1, 4096, 1024), (5, 1000, 1024), (16, 6000, 2048), (13, 200, 512), (3, 6, 3072),
                                    (3, 34, 3584), (8, 6000, 1152), (16, 300, 4480), (5, 64, 640)])
-def test_sparse_wave_per_tile_configs(sg, oracle, cfg, shape):
+def test_sparse_wave_per_tile_configs(sg, oracle, cfg, shape, k_chunks):
     """The wave-per-tile kernel (activations resident in LDS, every wave a whole tile over all of K, rotated K start):
-    more tiles than waves, fewer tiles than waves, ragged n and m, a single K stage, a K range of seven stages."""
+    more tiles than waves, fewer tiles than waves, ragged n and m, a single K stage, a single pair of stages, a K range
+    of seven stages; metadata by lines (pairs of stages running on across tile boundaries) and by pieces."""
     waves, row_tiles, depth, per_cu = cfg
     m, n, k = shape
     a8, vals, meta, b8, scale = oracle.make_sparse24_operands(m, n, k, seed=33)
     ref = sparse_reference(oracle, a8, vals, meta, scale)
-    t = sg.SgTuning(2, 1, waves, row_tiles, 1, depth, 8, 1, per_cu, 1)
+    t = sg.SgTuning(2, 1, waves, row_tiles, 1, depth, k_chunks, 1, per_cu, 1)
     rc, got = _run(sg, a8, vals, meta, scale, tuning=t)
     want = expect_sparse(m, n, k, record(2, 1, waves, row_tiles, 1, depth, 8, 1, per_cu, 1))
     assert rc == want, "library says %s, the resource rules say %d" % (sg.strerror(rc), want)
