@@ -729,7 +729,7 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
         // four waves per CU each stream whole tiles (4-33 % faster on ten shapes than refetching 4-8 KB of
         // activations with every 5 KB weight stage; at four rows and below the two are level)
         // (a K of whole 1024s gets its metadata by lines, which takes a pair ring next to the stages: at 9..16 rows and
-        // K = 4096 three stages with it, 9.0-9.1 us on 16 x 14336 x 4096, rather than four without, 9.3)
+        // K = 4096 three slots with it rather than four without - level to 2 % ahead on 16 x 14336 x 4096)
         const size_t x_res = (size_t)blocks * xu2 * 1024;
         for (int depth = 4; depth >= 2; depth--) {
             const size_t wave_bytes = k % 1024 == 0 ? (size_t)depth * 4096 + (size_t)(depth / 2 + 2) * 2048 : (size_t)depth * 5120;
@@ -744,7 +744,7 @@ static Config pick_sparse(int m, int n, int k, int cu_count) {
     }
     // Metadata by whole lines (launch_sparse_engine) costs a wave 4 KB of LDS more: with one-wave workgroups on
     // two-slot rings that is one workgroup less per CU, and up to 4 activation rows it does not pay (1 x 14336 x 4096
-    // 7.9 -> 8.0 us, where 32 x 14336 x 4096 on the same ring goes 12.7 -> 12.0 and 16 x 4096 x 14336 11.7 -> 10.2)
+    // 7.85 -> 7.83-8.0 us, where 32 x 14336 x 4096 on the same ring goes 12.3 -> 11.9 and 16 x 4096 x 14336 10.6 -> 10.1)
     if (m <= 4 && c.depth == 2 && c.waves == 1) c.ku = 1;
     return c;
 }

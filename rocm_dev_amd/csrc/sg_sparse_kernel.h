@@ -24,7 +24,7 @@
 // Metadata by whole cache lines (builds with PAIRS; K a multiple of 1024): 64 bytes per row and stage are half a
 // 128-byte line, so every metadata line is requested twice by the CU's L1, the second time as an L2 hit that waits
 // behind the misses around it - 48 requests per stage for 40 lines.  Asking once takes 10 % of the L1's requests away
-// and 1-4 % of the time on the 4096 x 14336 and 14336 x 4096 shapes (up to 12 % at 16 rows on K = 14336).  A PAIRS
+// and 0-5 % of the time on the 4096 x 14336 and 14336 x 4096 shapes (most at 16 rows on K = 14336).  A PAIRS
 // build takes its stages two at a time, (2P, 2P + 1), whose metadata is one aligned line per row: stage i carries,
 // next to its own values, the lines of rows 8h..8h+7 (h = i % 2) for the pair after its own, P = i / 2 + 1, into a ring of
 // DEPTH / 2 + 2 pair slots of its own; the first pair's lines go ahead of everything.  DMAs complete in order, so when
