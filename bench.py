@@ -110,6 +110,9 @@ def main():
                     help="only run the ingest probe (sg_debug_cu_ingest): what a CU takes in through direct-to-LDS loads from "
                          "beyond its XCD's L2 (cold), from inside it (hot), and from both at once out of the same or out of "
                          "different waves, with 16 and with 256 workgroups; prints a table, no JSON line")
+    ap.add_argument("--sparse", action="store_true",
+                    help="with --stamps --launch-shapes: the 2:4 GEMM (sg_sparse24_gemm on weights pruned and compressed here) "
+                         "instead of the dense one")
     ap.add_argument("--stamps", action="store_true",
                     help="only run the decode GEMMs (four projection shapes at M = --m) back to back from a HIP graph with "
                          "the library's per-workgroup time stamps switched on, and print where a launch period goes "
@@ -346,6 +349,17 @@ def main():
             args.m = m_
             copies = max(3, int(COLD_BYTES // (n * k)) + 1)
             wb = [quantize(torch.randn((n, k), device="cuda", dtype=torch.float32))[0] for _ in range(copies)]
+            if args.sparse:       # 2:4: prune and compress each weight buffer; a "copy" is then 0.625 of its dense bytes
+                packed = []
+                for w in wb:
+                    v = torch.empty((n, k // 2), device="cuda", dtype=torch.uint8)
+                    t = torch.empty((n, k // 8), device="cuda", dtype=torch.uint8)
+                    if lib.sg_sparse24_compress(w.data_ptr(), v.data_ptr(), t.data_ptr(), n, k, k, None) != 0:
+                        raise RuntimeError("sg_sparse24_compress failed")
+                    packed.append((v, t))
+                torch.cuda.synchronize()
+                wb = packed + [(v.clone(), t.clone()) for v, t in packed]
+                copies = len(wb)
             a8 = quantize(torch.randn((args.m, k), device="cuda", dtype=torch.float32))[0]
             d = torch.empty((args.m, n), device="cuda", dtype=torch.bfloat16)
             words = reps * 4096 * 8
@@ -357,10 +371,14 @@ def main():
                 with torch.cuda.graph(g, stream=side):
                     st = torch.cuda.current_stream().cuda_stream
                     for i in range(reps):
-                        rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(),
-                                                     args.m, n, k, k, st)
+                        if args.sparse:
+                            rc = lib.sg_sparse24_gemm(a8.data_ptr(), wb[i % copies][0].data_ptr(), wb[i % copies][1].data_ptr(),
+                                                      d.data_ptr(), one.data_ptr(), args.m, n, k, st)
+                        else:
+                            rc = lib.sg_skinny_gemm_auto(a8.data_ptr(), wb[i % copies].data_ptr(), d.data_ptr(), one.data_ptr(),
+                                                         args.m, n, k, k, st)
                         if rc != 0:
-                            raise RuntimeError("sg_skinny_gemm_auto: %s" % sg.strerror(rc))
+                            raise RuntimeError("%s: %s" % ("sg_sparse24_gemm" if args.sparse else "sg_skinny_gemm_auto", sg.strerror(rc)))
                 lib.sg_debug_stamps(None, 0)
                 ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 for _ in range(20):
@@ -388,12 +406,13 @@ def main():
                     "mhz": np.median((t[j, :, 6].astype(np.int64) - t[j, :, 5].astype(np.int64)) / np.maximum(end[j] - ent[j], tick))})
             med = {key: float(np.median([r[key] for r in rows])) for key in rows[0]}
             t_choice, _ = sg.skinny_gemm_choice(args.m, n, k)
+            what = "2:4, the library's choice" if args.sparse else sg.api.tuning_as_dict(t_choice)
             print("%-18s %5d x %5d  grid %4d  event-pair period %.2f | period %.2f = gap %.2f + span %.2f | entry spread %.2f | "
                   "workgroup (median): prologue issue %.2f, first stage landed %.2f (max %.2f), streaming %.2f, reduce+store %.2f, "
                   "total %.2f (max %.2f) | last end - median end %.2f | shader clock %.0f MHz | %s"
                   % (name, n, k, grid, period_ev, med["period"], med["gap"], med["span"], med["spread"], med["issue"], med["land_med"],
                      med["land_max"], med["stream"], med["epi"], med["wg_med"], med["wg_max"], med["tail"], med["mhz"],
-                     sg.api.tuning_as_dict(t_choice)), flush=True)
+                     what), flush=True)
             # does the finish time depend on the XCD?  per XCC_ID: median and latest workgroup end after the launch's first entry
             xcc = (t[4:, :, 7] >> np.uint64(32)).astype(np.int64) & 0xF
             rel_end = end[4:] - ent[4:].min(axis=1, keepdims=True)
@@ -402,6 +421,12 @@ def main():
                 sel = rel_end[xcc == x]
                 line.append("xcc%d %.2f/%.2f" % (x, float(np.median(sel)), float(np.median(np.where(xcc == x, rel_end, 0).max(axis=1)))))
             print("         workgroup end after first entry, median / median-of-latest per XCD: " + "  ".join(line), flush=True)
+            # are the late workgroups the same ones in every launch (their share of the work, their CU) or any (queueing)?
+            corr = [float(np.corrcoef(rel_end[j], rel_end[j + 1])[0, 1]) for j in range(rel_end.shape[0] - 1)]
+            print("         workgroup end after first entry: median %.2f, 90th percentile %.2f, latest %.2f; correlation of a "
+                  "workgroup's end between consecutive launches %.2f"
+                  % (float(np.median(rel_end)), float(np.percentile(rel_end, 90)), float(np.median(rel_end.max(axis=1))),
+                     float(np.median(corr))), flush=True)
             del wb, buf
         return
 

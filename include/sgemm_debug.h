@@ -14,7 +14,7 @@ extern "C" {
 #endif
 
 /* Profiling aid, no counterpart in the reference.  While a buffer is set, every launch of the LDS-ring GEMM
- * kernels (per-tile and persistent) and of the mid-batch GEMM kernel takes the next grid * 8 words of it and each workgroup leaves eight 64-bit
+ * kernels (per-tile and persistent), of the mid-batch GEMM kernel and of the 2:4 kernels takes the next grid * 8 words of it and each workgroup leaves eight 64-bit
  * words there when it is done: [0] kernel entry, [1] prologue DMAs issued, [2] first stage landed, [3] last stage
  * consumed, [4] outputs stored and acknowledged - 10 ns ticks of the device's constant 100 MHz clock -
  * [5], [6] shader clock at entry and end, [7] XCC_ID << 32 | HW_ID.  Launches that no longer fit leave nothing.

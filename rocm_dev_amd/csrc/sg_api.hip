@@ -690,6 +690,7 @@ static int launch_sparse_engine(const Config& c, StreamArgs a, const uint8_t* me
         if (int rc = get_device_info(&dev)) return rc;
         size_t grid = (size_t)dev->cu_count * c.persist;
         if (grid > tiles) grid = tiles;
+        a.stamps = take_stamps((unsigned)grid);
         sa.g = a;
         return launch_sparse_wavetile(c.rg, xu2, c.depth, pairs, sa, (unsigned)grid, (unsigned)c.waves * 64, lds_wt, stream);
     }
@@ -700,6 +701,7 @@ static int launch_sparse_engine(const Config& c, StreamArgs a, const uint8_t* me
     const size_t lds_pairs = (size_t)c.waves * (c.depth * (stage - (size_t)c.rg * 1024) + pair_ring) + 8192;
     pairs = pairs && lds_pairs <= 159 * 1024;
     if (pairs) lds = lds_pairs;
+    a.stamps = take_stamps((unsigned)(tiles * c.split_k));
     sa.g = a;
     return launch_sparse(c.mt, c.rg, xu2, c.depth, pairs, sa, (unsigned)(tiles * c.split_k), (unsigned)c.waves * 64, lds, stream);
 }

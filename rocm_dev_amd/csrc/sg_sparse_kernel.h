@@ -67,6 +67,8 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // [wave][DEPTH][stage] (PAIRS: + [pair slot][rg][2 KB])
     __shared__ unsigned arrival;
     const StreamArgs& a = sa.g;
+    Stamps stamps;
+    stamps.begin();
 
     constexpr int PER_STAGE = RG * 5 + XU2;   // DMA instructions per stage
     constexpr int W_TILE = PAIRS ? 4096 : 5120;   // a row tile's part of a stage: 4 KB values [| 1 KB metadata]
@@ -225,9 +227,11 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
     if (mine >= DEPTH) {
 #pragma unroll
         for (int d = 0; d < DEPTH; d++) issue(d);
+        stamps.mark(1);
         int i = 0;
         for (; i + DEPTH < mine; i++) {
             wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            if (i == 0) stamps.mark(2);
             consume(i);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
@@ -237,13 +241,17 @@ __global__ void __launch_bounds__(sparse_launch_bound(MT, RG)) sparse24_gemm_ker
         drain_ring<0, DEPTH, PER_STAGE>(consume, i);
     } else {
         for (int i = 0; i < mine; i++) issue(i);
+        stamps.mark(1);
         wait_vmcnt<0>();
+        stamps.mark(2);
         for (int i = 0; i < mine; i++) consume(i);
     }
+    stamps.mark(3);
 
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __syncthreads();
     finish_tile<RG, MT>(a, acc, reinterpret_cast<f32x4*>(ring), &arrival, tile_m, tile_n, split, m0, n0);
+    stamps.end(a);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -260,6 +268,8 @@ template <int RG, int XU2, int DEPTH, bool TAIL, bool PAIRS>
 __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_kernel(const SparseArgs sa) {
     extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];  // X[stages][XU2 KB] | [wave][sparse_wave_bytes] | 8 KB
     const StreamArgs& a = sa.g;
+    Stamps stamps;
+    stamps.begin();
 
     constexpr int PER_STAGE = RG * 5;
     constexpr int W_TILE = PAIRS ? 4096 : 5120;
@@ -419,6 +429,7 @@ __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_k
         }
     }
     for (int d = 0; d < pro; d++) issue(d);
+    stamps.mark(1);
     if (x_issued > 0) wait_vmcnt_upto(pro * PER_STAGE);
     __syncthreads();
 
@@ -426,6 +437,7 @@ __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_k
         int i = 0;
         for (; i + DEPTH < total; i++) {
             wait_vmcnt<(DEPTH - 1) * PER_STAGE>();
+            if (i == 0) stamps.mark(2);
             consume(i);
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
@@ -440,11 +452,14 @@ __global__ void __launch_bounds__(RG == 4 ? 512 : 1024) sparse24_gemm_wavetile_k
         drain_ring<0, DEPTH, PER_STAGE>(consume_and_close, i);
     } else {
         wait_vmcnt<0>();
+        stamps.mark(2);
         for (int i = 0; i < total; i++) {
             consume(i);
             after_consume();
         }
     }
+    stamps.mark(3);   // (the tiles' stores are part of the streaming phase here: every wave stores as it goes)
+    stamps.end(a);
 }
 
 
