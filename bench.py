@@ -347,6 +347,11 @@ def main():
             jobs = [(s, *[int(v) for v in s.lower().split("x")]) for s in args.launch_shapes]
         for name, m_, n, k in jobs:
             args.m = m_
+            if args.record and not args.sparse:     # a given tuning record instead of the library's choice
+                import ctypes
+                forced = sg.SgTuning(*args.record)
+                if lib.sg_tuning_set(m_, n, k, ctypes.byref(forced)) != 0:
+                    sys.exit("bench.py: --record is not a valid tuning record")
             copies = max(3, int(COLD_BYTES // (n * k)) + 1)
             wb = [quantize(torch.randn((n, k), device="cuda", dtype=torch.float32))[0] for _ in range(copies)]
             if args.sparse:       # 2:4: prune and compress each weight buffer; a "copy" is then 0.625 of its dense bytes
