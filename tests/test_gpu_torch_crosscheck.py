@@ -2,6 +2,7 @@
 output against torch's dequantise-to-fp32 matmul (rocBLAS, a different summation order, no code shared with
 the library or the oracle), and against torch._scaled_mm (hipBLASLt's own FP8 path) where this torch build
 has it.  The oracle-based tests cover slices of these shapes; this covers every tile of them."""
+import math
 import random
 
 import pytest
@@ -161,3 +162,106 @@ def test_against_scaled_mm(sg, m, n, k):
     assert sg.skinny_gemm_fastpath(A, B, D, S) == 0
     torch.cuda.synchronize()
     assert _metric(D, ref) <= GEMM_TOL
+
+
+def _guarded_output(m, n):
+    """An m x n bf16 output inside a larger buffer: eight rows of a sentinel value either side (16-byte aligned for
+    every even n), NaN where the result goes."""
+    whole = torch.full((m + 16, n), 12345.0, dtype=torch.bfloat16, device="cuda")
+    whole[8:m + 8] = float("nan")
+    return whole, whole[8:m + 8]
+
+
+def _guards_intact(whole, m):
+    return bool((whole[:8] == 12345.0).all()) and bool((whole[m + 8:] == 12345.0).all())
+
+
+def _random_case(seed):
+    """m 1..700, n 2..60000 (log-uniform), k 2048..32768 in steps of 16..512, a third with padded weight rows."""
+    rng = random.Random(seed)
+    r = rng.random()
+    m = rng.randint(1, 32) if r < 0.4 else (rng.randint(33, 256) if r < 0.8 else rng.randint(257, 700))
+    g = rng.choice([16, 64, 128, 128, 256, 256, 512])
+    k = g * int(math.exp(rng.uniform(math.log(2048 // g), math.log(32768 // g))))
+    n = 2 * int(math.exp(rng.uniform(0.0, math.log(30000))))
+    while n * k > (256 << 20):
+        n //= 2
+    n = max(2, n - n % 2)
+    pad = 16 * rng.randint(1, 4) if rng.random() < 0.3 else 0
+    kind = rng.choice(["fast", "fast", "rowcol", "bf16act", "sparse"])
+    if kind == "sparse" and (k % 128 or m > 64):
+        kind = "fast"
+    return kind, m, n, k, pad
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_shapes_between_guard_rows(sg, seed):
+    """Seeded random shapes through the entry points that choose their own launch, the output between guard rows:
+    nothing outside the m x n result is written, every element of it is, the result matches torch's unrounded fp32
+    matmul (the row and column factors divided out again, so that the metric's floor is the same for every column),
+    the caller-owned workspace gives the library-owned one's bits, and the fused activation quantisation those of
+    encode + GEMM."""
+    kind, m, n, k, pad = _random_case(seed)
+    gen = torch.Generator(device="cuda").manual_seed(7919 * seed + 1)
+    a = torch.randn((m, k), generator=gen, device="cuda")
+    w = torch.randn((n, k), generator=gen, device="cuda")
+    sa, sb = a.abs().max() / 448.0, w.abs().max() / 448.0
+    A = (a / sa).to(torch.float8_e4m3fn)
+    padded = torch.full((n, k + pad), 0x7f, dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn)   # NaN codes in the padding
+    padded[:, :k] = (w / sb).to(torch.float8_e4m3fn)
+    B = padded[:, :k]
+    del a, w
+    S = (sa * sb).reshape(1).float()
+    whole, D = _guarded_output(m, n)
+    case = (kind, m, n, k, pad)
+    if kind == "sparse":
+        codes = B.contiguous().view(torch.uint8)
+        vals = torch.empty((n, k // 2), dtype=torch.uint8, device="cuda")
+        meta = torch.empty((n, k // 8), dtype=torch.uint8, device="cuda")
+        assert sg.sparse24_compress(codes, vals, meta) == 0
+        assert sg.sparse24_gemm(A, vals, meta, D, S) == 0, case
+        torch.cuda.synchronize()
+        mag = (codes & 0x7f).to(torch.int16).view(n, k // 4, 4)
+        key = mag * 4 + (3 - torch.arange(4, device="cuda", dtype=torch.int16))
+        keep = torch.zeros_like(mag, dtype=torch.bool)
+        keep.scatter_(2, key.topk(2, dim=2).indices, True)
+        pruned = torch.where(keep.view(n, k), codes, torch.zeros_like(codes)).view(torch.float8_e4m3fn)
+        assert _guards_intact(whole, m), case
+        assert _metric(D, _dequant_matmul(A, pruned, S, rounded=False)) <= GEMM_TOL, case
+        return
+    if kind == "bf16act":
+        X = (torch.randn((m, k), generator=gen, device="cuda") * 3).bfloat16()
+        cs = torch.rand(n, generator=gen, device="cuda") + 0.5
+        rs_out = torch.empty(m, dtype=torch.float32, device="cuda")
+        assert sg.skinny_gemm_bf16act(X, B, D, S, cs, rs_out) == 0, case
+        Q = torch.empty((m, k), dtype=torch.uint8, device="cuda")
+        scales = torch.empty(m, dtype=torch.float32, device="cuda")
+        assert sg.fp8_encode_rows(X, Q, scales) == 0
+        whole2, D2 = _guarded_output(m, n)
+        assert sg.skinny_gemm_rowcol(Q.view(torch.float8_e4m3fn), B, D2, S, scales, cs) == 0, case
+        torch.cuda.synchronize()
+        assert _guards_intact(whole, m) and _guards_intact(whole2, m), case
+        assert torch.equal(D.view(torch.int16), D2.view(torch.int16)) and torch.equal(scales, rs_out), case
+        ref = _dequant_matmul(Q.view(torch.float8_e4m3fn), B, S, rounded=False)
+        assert _metric(D.float() / cs[None, :] / scales[:, None], ref) <= GEMM_TOL, case
+        return
+    if kind == "rowcol":
+        rs = torch.rand(m, generator=gen, device="cuda") * 1.5 + 0.5
+        cs = torch.rand(n, generator=gen, device="cuda") * 1.5 + 0.5
+        assert sg.skinny_gemm_rowcol(A, B, D, S, rs, cs) == 0, case
+        torch.cuda.synchronize()
+        assert _guards_intact(whole, m), case
+        assert _metric(D.float() / (rs[:, None] * cs[None, :]), _dequant_matmul(A, B, S, rounded=False)) <= GEMM_TOL, case
+        return
+    assert sg.skinny_gemm_fastpath(A, B, D, S) == 0, case
+    need = sg.workspace_query(m, n, k)
+    ws = None
+    if need:
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        sg.workspace_init(ws)
+    whole2, D2 = _guarded_output(m, n)
+    assert sg.skinny_gemm_auto_ws(A, B, D2, S, ws) == 0, case
+    torch.cuda.synchronize()
+    assert _guards_intact(whole, m) and _guards_intact(whole2, m), case
+    assert torch.equal(D.view(torch.int16), D2.view(torch.int16)), case
+    assert _metric(D, _dequant_matmul(A, B, S, rounded=False)) <= GEMM_TOL, case
